@@ -25,10 +25,16 @@ def _dogudra():
     return DogudraForCausalLM
 
 
+def _kitonex():
+    from .kitonex import KitonexForCausalLM
+    return KitonexForCausalLM
+
+
 REGISTRY = {
     "qwen3": _qwen, "qwen2": _qwen, "qwen3forcausallm": _qwen, "qwen2forcausallm": _qwen,
     "mobupel": _mobupel, "mobupelforcausallm": _mobupel,
     "dogudra": _dogudra, "dogudraforcausallm": _dogudra,
+    "kitonex": _kitonex, "kitonexforcausallm": _kitonex,
 }
 
 

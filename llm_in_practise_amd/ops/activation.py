@@ -74,3 +74,12 @@ def clipped_glu(z: torch.Tensor, limit: float) -> torch.Tensor:
     if use_seq(z):
         return native_seq().ff_act(z.contiguous(), 1, limit)
     return ref.clipped_glu(z, limit)
+
+
+def silu_glu(z: torch.Tensor) -> torch.Tensor:
+    """``z = [gate | up]``: ``silu(gate) * up``."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(z):
+        return native_seq().ff_act(z.contiguous(), 2, 0.0)
+    return ref.silu_glu(z)

@@ -201,3 +201,46 @@ def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, 
         return native_seq().latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, nsplit,
                                              sb.desc, sb.tiles)
     return ref.latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, sb)
+
+
+def distance_bias_table(rel: torch.Tensor, far: float, distances: int) -> torch.Tensor:
+    """A learned bias per (distance bucket, head) ``rel`` ``[B, H]`` spread out by distance: float ``[H, distances]``
+    whose entry ``[h, n]`` is ``rel[bucket(n), h]``.  The first half of the buckets are exact distances; the second
+    half grow logarithmically up to ``far``: ``bucket(n) = n`` below ``B/2``, else
+    ``min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(far / (B/2)) * (B - B/2)))``."""
+    import math
+    B = rel.shape[0]
+    half = B // 2
+    ids = [n if n < half else min(B - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (B - half))))
+           for n in range(distances)]
+    return rel.float()[torch.tensor(ids, dtype=torch.long, device=rel.device)].t().contiguous()
+
+
+def qk_norm_store(u: torch.Tensor, nq: int, nk: int, q_weight: torch.Tensor, k_weight: torch.Tensor,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, v_first: torch.Tensor | None, lam, eps: float,
+                  sb) -> torch.Tensor:
+    """The step's ``[q | k | v]`` rows ``u`` ``[T, nq + nk + nv]`` on their way into attention: q and k are RMS-normed
+    over their whole width (all heads at once, weights ``[nq]`` / ``[nk]``), the normed k goes to ``k_cache``
+    ``[slots, max_len, nk]`` at each token's slot and position, v to ``v_cache`` — with ``v_first`` (another layer's
+    value cache, same shape) as ``(1 - lam) v + lam v_first[slot, pos]`` (``lam`` a one-element float tensor).
+    Returns the normed q ``[T, nq]``."""
+    from ._native import native_seq, use_seq
+    if use_seq(u):
+        return native_seq().qk_norm_store(u, nq, nk, q_weight, k_weight, k_cache, v_cache, v_first, lam, eps, sb.desc)
+    return ref.qk_norm_store(u, nq, nk, q_weight, k_weight, k_cache, v_cache, v_first, lam, eps, sb)
+
+
+def biased_attention(q, k_cache, v_cache, bias: torch.Tensor | None, heads: int, kv_heads: int, scale: float, sb,
+                     block: int = 0, sink: float | None = None, nsplit: int = 1):
+    """Causal grouped-query softmax attention over a slot-indexed cache with three optional parts:
+    ``bias`` float ``[H, ND]`` adds ``bias[h, min(i - j, ND - 1)]`` to the scaled score of query ``i`` and key ``j``
+    (``scale`` does not multiply it); ``block > 0`` lets a query see only keys of its own run of ``block`` positions
+    (runs counted from the sequence's position 0); ``sink`` adds one key of that score and no value to every
+    softmax (``0.0``: one is added to the denominator).  ``q`` ``[T, H*dk]`` for the step's packed tokens; the caches
+    ``[slots, max_len, G*dk | G*dv]`` already hold the step's rows.  Returns ``[T, H*dv]``; scores and weights are
+    float.  ``nsplit`` cuts each query's keys into that many independent sweeps (decode)."""
+    from ._native import native_seq, use_seq
+    if use_seq(q):
+        return native_seq().biased_attention(q, k_cache, v_cache, bias, heads, kv_heads, scale, block,
+                                             sink is not None, float(sink or 0.0), nsplit, sb.desc, sb.tiles)
+    return ref.biased_attention(q, k_cache, v_cache, bias, heads, kv_heads, scale, block, sink, sb)

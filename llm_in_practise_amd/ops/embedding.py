@@ -134,3 +134,15 @@ def embed_pair(tokens: torch.Tensor, table: torch.Tensor, pair_table: torch.Tens
         return tuple(native_seq().embed_pair(tokens.reshape(-1).long().contiguous(), table, pair_table, prev, scale,
                                              mul_prev, mul_cur, sb.desc, sb.live))
     return ref.embed_pair(tokens, table, pair_table, prev, scale, mul_prev, mul_cur, sb)
+
+
+def embed_learned(tokens: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, pos_table: torch.Tensor,
+                  streams: int = 1) -> torch.Tensor:
+    """Token row plus a learned position row (not scaled), as ``streams`` equal float copies ``[T, streams, width]``:
+    the residual streams of a model with several of them (one for a plain residual)."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(table):
+        return native_seq().embed_learned(tokens.reshape(-1).long().contiguous(), positions.reshape(-1).int().contiguous(),
+                                          table, pos_table, streams)
+    return ref.embed_learned(tokens, positions, table, pos_table, streams)

@@ -138,29 +138,51 @@ def moe_combine(ys: torch.Tensor, d: Dispatch, w: torch.Tensor, base: torch.Tens
 
 
 # ------------------------------------------------------------------ serving: grouped routing, identity experts
+ROUTE_SIGMOID, ROUTE_TOP2, ROUTE_NORMALIZE = 1, 2, 4
+
+
+def _route_kind(score: str, group_rank: str, normalize: bool) -> int:
+    if score not in ("softmax", "sigmoid") or group_rank not in ("max", "top2"):
+        raise ValueError(f"routing: unknown score {score!r} or group rank {group_rank!r}")
+    return (ROUTE_SIGMOID if score == "sigmoid" else 0) | (ROUTE_TOP2 if group_rank == "top2" else 0) | \
+        (ROUTE_NORMALIZE if normalize else 0)
+
+
 def route_grouped(logits: torch.Tensor, correction: torch.Tensor | None, top: int, groups: int = 1, keep: int = 1,
-                  scale: float = 1.0):
+                  scale: float = 1.0, score: str = "softmax", group_rank: str = "max", normalize: bool = False):
     """Float router logits ``[T, n]`` -> ``(expert ids int32 [T, top], weights float [T, top])``.  Scores are the
-    softmax over all ``n`` outputs; the choice is made on ``score + correction``, restricted to the ``keep`` best of
-    ``groups`` equal runs of neighbouring outputs (a run's rank is its largest choice value); the weights are the
-    plain scores times ``scale``, not renormalised."""
+    softmax over all ``n`` outputs (``score="sigmoid"``: each output's own sigmoid); the choice is made on
+    ``score + correction``, restricted to the ``keep`` best of ``groups`` equal runs of neighbouring outputs (a run's
+    rank is its largest choice value, or with ``group_rank="top2"`` the sum of its two largest); the weights are the
+    plain scores times ``scale``, with ``normalize`` first divided by their sum over the chosen (+ 1e-20)."""
     from . import reference as ref
     from ._native import native_seq, use_seq
+    kind = _route_kind(score, group_rank, normalize)
     if use_seq(logits):
-        idx, w = native_seq().route_grouped(logits.contiguous(), correction, top, groups, keep, scale)
+        idx, w = native_seq().route_grouped(logits.contiguous(), correction, top, groups, keep, scale, kind)
         return idx, w
-    return ref.route_grouped(logits, correction, top, groups, keep, scale)
+    return ref.route_scored(logits, correction, top, groups, keep, scale, score == "sigmoid", group_rank == "top2",
+                            normalize)
 
 
 def route_tokens(h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, groups: int = 1,
-                 keep: int = 1, scale: float = 1.0):
+                 keep: int = 1, scale: float = 1.0, score: str = "softmax", group_rank: str = "max",
+                 normalize: bool = False, extra: int = 0):
     """:func:`route_grouped` on the logits ``h @ router^T`` (``router`` float ``[n, W]``; the products accumulate in
-    float whatever ``h``'s dtype).  On the GPU product and routing are one kernel."""
+    float whatever ``h``'s dtype).  On the GPU product and routing are one kernel.  The last ``extra`` rows of
+    ``router`` are not routed: their products come back raw as a third result, float ``[T, extra]`` (small per-token
+    gates that read the same input ride along)."""
+    from . import reference as ref
     from ._native import native_seq, use_seq
+    kind = _route_kind(score, group_rank, normalize)
     if use_seq(h):
-        idx, w = native_seq().route_fused(h, router, correction, top, groups, keep, scale)
-        return idx, w
-    return route_grouped(h.float() @ router.t(), correction, top, groups, keep, scale)
+        idx, w, ex = native_seq().route_fused(h, router, correction, top, groups, keep, scale, kind, extra)
+        return (idx, w, ex) if extra else (idx, w)
+    z = h.float() @ router.t()
+    n = router.shape[0] - extra
+    idx, w = ref.route_scored(z[:, :n], correction, top, groups, keep, scale, score == "sigmoid", group_rank == "top2",
+                              normalize)
+    return (idx, w, z[:, n:].contiguous()) if extra else (idx, w)
 
 
 PAD_ROWS = 128      # sorted path: an expert's products run over a multiple of this many rows (0: exactly its rows)
@@ -168,8 +190,10 @@ PAD_ROWS = 128      # sorted path: an expert's products run over a multiple of t
 
 def moe_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor,
                     weights: torch.Tensor, limit: float, shared: torch.Tensor | None = None,
-                    few_tokens: bool = False) -> torch.Tensor:
-    """Weighted sum of the chosen clipped-GLU experts' outputs, float ``[T, W]``.  ``w_gate_up`` ``[E, 2, F, W]``,
+                    few_tokens: bool = False, act: str = "clipped", shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+    """Weighted sum of the chosen GLU experts' outputs, float ``[T, W]`` (``act="clipped"``: the clipped GLU with
+    ``limit``; ``act="silu"``: ``silu(gate) * up``, ``limit`` unused; ``shared_gate`` float ``[T]``: the shared
+    expert's output is multiplied by its sigmoid).  ``w_gate_up`` ``[E, 2, F, W]``,
     ``w_down`` ``[E, W, F]``; ids ``>= E`` are identity experts (their output is ``h``); ``shared`` ``[T, W]`` is
     added.  ``few_tokens`` (decode steps, captured graphs): every (token, expert) pair streams its expert's rows in
     two kernels with no sort and no host round trip.  Otherwise rows are sorted by expert, every expert runs one
@@ -177,12 +201,16 @@ def moe_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tens
     multiple of ``PAD_ROWS`` rows), and a kernel combines."""
     from . import reference as ref
     from ._native import native_seq, use_seq
-    from .activation import clipped_glu
+    from .activation import clipped_glu, silu_glu
+    if act not in ("clipped", "silu"):
+        raise ValueError(f"experts: unknown activation {act!r}")
+    mode = 1 if act == "clipped" else 2
+    glu = (lambda z: clipped_glu(z, limit)) if mode == 1 else silu_glu
     T, W = h.shape
     E, _, F_, _ = w_gate_up.shape
     top = idx.shape[1]
     if use_seq(h) and few_tokens:
-        return native_seq().moe_pairs(h.contiguous(), w_gate_up, w_down, idx, weights, shared, limit)
+        return native_seq().moe_pairs(h.contiguous(), w_gate_up, w_down, idx, weights, shared, limit, mode, shared_gate)
     flat = idx.reshape(-1).long()
     order = torch.sort(flat, stable=True).indices
     counts = torch.bincount(flat, minlength=E).tolist()[:E]
@@ -200,15 +228,17 @@ def moe_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tens
         if n:
             m = min(-(-n // pad) * pad, rows + pad - a) if pad else n
             z = xs[a:a + m] @ w_gate_up[e].reshape(2 * F_, W).t()
-            torch.mm(clipped_glu(z, limit), w_down[e].t(), out=ys[a:a + m])
+            torch.mm(glu(z), w_down[e].t(), out=ys[a:a + m])
             a += n
     pos = torch.empty_like(order)
     pos[order] = torch.arange(order.numel(), device=order.device)
     if use_seq(h):
-        return native_seq().moe_combine_sorted(ys, pos.contiguous(), idx, weights, h.contiguous(), shared, E)
+        return native_seq().moe_combine_sorted(ys, pos.contiguous(), idx, weights, h.contiguous(), shared, E, shared_gate)
     pos = pos.view(T, top)
     own = idx.long() >= E
     picked = torch.where(own[..., None], h.float()[:, None, :], ys.float()[pos.clamp(max=max(rows - 1, 0))]
                          if rows else h.float()[:, None, :].expand(T, top, W))
     out = (picked * weights[..., None]).sum(1)
-    return out if shared is None else out + shared.float()
+    if shared is None:
+        return out
+    return out + (shared.float() if shared_gate is None else shared.float() * torch.sigmoid(shared_gate)[:, None])

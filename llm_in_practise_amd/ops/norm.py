@@ -182,3 +182,16 @@ def gate_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, part
     if use_seq(y):
         return native_seq().gate_group_norm(y, z, weight, parts, eps)
     return ref.gate_group_norm(y, z, weight, parts, eps)
+
+
+def hyper_mix_norm(X: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, out: torch.Tensor | None,
+                   read: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype) -> torch.Tensor:
+    """A sublayer's exit and the next one's entry over ``S`` residual streams ``X`` (float ``[T, S, W]``, in place):
+    with the sublayer's output ``y`` ``[T, W]``, all streams at once from the old ones
+    ``X_t <- sum_s mix[s, t] X_s + out[t] y``; then returns ``rmsnorm(sum_s read[s] X_s) * weight`` in ``dtype``, the
+    next sublayer's input (``read`` all ones: the sum of the streams, for the model's last norm).  ``y = None`` only
+    reads (the first sublayer's entry).  One stream with ``mix = out = read = 1`` is the plain pre-norm residual."""
+    from ._native import native_seq, use_seq
+    if use_seq(X):
+        return native_seq().hyper_mix_norm(X, y, mix, out, read, weight, eps, dtype == torch.bfloat16)
+    return ref.hyper_mix_norm(X, y, mix, out, read, weight, eps, dtype)

@@ -392,16 +392,7 @@ def latent_attention(qa, q, cache, gate, inv_freq, H: int, dn: int, dims: int, s
 
 
 def route_grouped(z, corr, top: int, groups: int, keep: int, scale: float):
-    T, n = z.shape
-    s = torch.softmax(z.float(), -1)
-    ch = s + corr if corr is not None else s.clone()
-    if groups > 1 and keep < groups:
-        best = ch.view(T, groups, n // groups).max(-1).values
-        kept = torch.zeros(T, groups, dtype=torch.bool, device=z.device)
-        kept.scatter_(1, best.topk(keep, -1).indices, True)
-        ch = ch.masked_fill(~kept.repeat_interleave(n // groups, 1), float("-inf"))
-    idx = ch.topk(top, -1).indices
-    return idx.int(), s.gather(1, idx) * scale
+    return route_scored(z, corr, top, groups, keep, scale, False, False, False)
 
 
 def clipped_glu(z, limit: float):
@@ -413,3 +404,82 @@ def clipped_glu(z, limit: float):
 
 def gelu_tanh(z):
     return F.gelu(z.float(), approximate="tanh").to(z.dtype)
+
+
+# ---- pre-normed layers over several residual streams, biased block attention with a sink, sigmoid routing
+def embed_learned(tok, pos, table, pos_table, streams: int):
+    x = table[tok.reshape(-1).long()].float() + pos_table[pos.reshape(-1).long()].float()
+    return x[:, None, :].repeat(1, streams, 1)
+
+
+def hyper_mix_norm(X, y, mix, out, read, w, eps: float, dtype):
+    if y is not None:
+        X.copy_(torch.einsum("st,nsw->ntw", mix, X) + out[None, :, None] * y.float()[:, None, :])
+    u = (read[None, :, None] * X).sum(1)
+    return (_unit_rms(u, eps) * w).to(dtype)
+
+
+def qk_norm_store(u, nq: int, nk: int, qw, kw, kc, vc, v_first, lam, eps: float, sb):
+    q = (_unit_rms(u[:, :nq].float(), eps) * qw).to(u.dtype)
+    k = (_unit_rms(u[:, nq:nq + nk].float(), eps) * kw).to(u.dtype)
+    v = u[:, nq + nk:]
+    if v_first is not None:
+        first = v_first.view(-1, v_first.shape[2])[sb.cache_idx].float()
+        v = ((1.0 - lam) * v.float() + lam * first).to(u.dtype)
+    kc.view(-1, nk).index_copy_(0, sb.cache_idx, k)
+    vc.view(-1, vc.shape[2]).index_copy_(0, sb.cache_idx, v.to(vc.dtype))
+    return q
+
+
+def biased_attention(q, kc, vc, bias, H: int, G: int, scale: float, block: int, sink, sb):
+    T = q.shape[0]
+    dk, dv = q.shape[1] // H, vc.shape[2] // G
+    rep = H // G
+    out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        a, e = off[b], off[b + 1]
+        L = pos0[b] + e - a
+        kk = kc[slot, :L].float().view(L, G, dk).repeat_interleave(rep, 1)      # [L, H, dk]
+        vv = vc[slot, :L].float().view(L, G, dv).repeat_interleave(rep, 1)
+        sc = torch.einsum("thd,lhd->htl", q[a:e].float().view(e - a, H, dk), kk) * scale
+        qp = pos0[b] + torch.arange(e - a, device=q.device)
+        kp = torch.arange(L, device=q.device)
+        dist = qp[:, None] - kp[None, :]
+        vis = dist >= 0
+        if block > 0:
+            vis &= (qp[:, None] // block) == (kp[None, :] // block)
+        if bias is not None:
+            sc = sc + bias[:, dist.clamp(0, bias.shape[1] - 1)]
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        m = sc.max(-1, keepdim=True).values
+        if sink is not None:
+            m = m.clamp(min=float(sink))
+        w = torch.exp(sc - m)
+        den = w.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(float(sink) - m)
+        out[a:e] = torch.einsum("htl,lhd->thd", w / den, vv).reshape(e - a, H * dv)
+    return out.to(q.dtype)
+
+
+def route_scored(z, corr, top: int, groups: int, keep: int, scale: float, sigmoid: bool, top2: bool, normalize: bool):
+    T, n = z.shape
+    s = torch.sigmoid(z.float()) if sigmoid else torch.softmax(z.float(), -1)
+    ch = s + corr if corr is not None else s.clone()
+    if groups > 1 and keep < groups:
+        per = ch.view(T, groups, n // groups)
+        rank = per.topk(min(2, n // groups), -1).values.sum(-1) if top2 else per.max(-1).values
+        kept = torch.zeros(T, groups, dtype=torch.bool, device=z.device)
+        kept.scatter_(1, rank.topk(keep, -1).indices, True)
+        ch = ch.masked_fill(~kept.repeat_interleave(n // groups, 1), float("-inf"))
+    idx = ch.topk(top, -1).indices
+    w = s.gather(1, idx)
+    if normalize:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx.int(), w * scale
+
+
+def silu_glu(z):
+    F_ = z.shape[-1] // 2
+    return (F.silu(z[..., :F_].float()) * z[..., F_:].float()).to(z.dtype)
