@@ -8,28 +8,45 @@
 // rows).  Pass 2 merges the splits, normalises, mixes the heads with talk, applies the sigmoid output gate and writes
 // the activation type.  Scores, weights and U are float.  One wave per (token, head, split): lanes own keys for
 // q.k (each lane one key's full dot product, q broadcast from LDS), then own value columns for w.V.
+//
+// The same sweeps serve plain grouped-query attention (GQA = true): a query head meets only the values of its own kv
+// head, and three optional parts change which keys count and how: a float bias per (head, distance) added to the
+// scaled score, a block mask (a query sees only the keys of its own run of `block` positions, counted from the
+// sequence's position 0), and a sink (one more key of a fixed score without a value in every softmax).  With one key
+// split the matrix-core sweep normalises and writes the activation type itself; otherwise k_gqa_merge does.
 #include "seq_common.h"
 
 using namespace lipa;
 
+// what GQA = true adds to a sweep
+struct GqaExtra {
+  const float* bias;   // [H, nd] or null: bias[h][min(i - j, nd - 1)], in natural-log units
+  int nd;
+  int block;           // 0: every earlier key; > 0: keys of the query's own block
+  int sink;            // 1: a key of score sink_logit and no value
+  float sink_logit;
+  void* out;           // [T, H * dv] in the activation type, written when nsplit == 1 (matrix-core sweep)
+};
+
 constexpr int MAXC = 16;   // value columns per lane: G * dv <= 64 * MAXC
 
-template <typename T>
+template <typename T, bool GQA>
 __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ q, int ldq, const T* __restrict__ kc,
                                                           const T* __restrict__ vc, float* __restrict__ pm,
                                                           float* __restrict__ pl, float* __restrict__ pu, int H, int G,
                                                           int dk, int dv, int ldk, int ldv, int max_len, int nsplit,
-                                                          float scale, SeqDesc d) {
+                                                          float scale, SeqDesc d, GqaExtra x) {
   extern __shared__ float sq[];
   const int t = blockIdx.x, g = blockIdx.y, z = blockIdx.z, lane = threadIdx.x;
   const int s = d.tok_seq[t], p = d.tok_pos[t], slot = d.slots[s];
-  const int kh = g / (H / G), GV = G * dv;
+  const int kh = g / (H / G), GV = GQA ? dv : G * dv;
   for (int i = lane; i < dk; i += 64) sq[i] = (float)q[(size_t)t * ldq + g * dk + i];
   __syncthreads();
-  const int nkeys = p + 1, per = (nkeys + nsplit - 1) / nsplit;
-  const int j0 = z * per, j1 = min(nkeys, j0 + per);
+  const int lo = (GQA && x.block > 0) ? (p / x.block) * x.block : 0;
+  const int nkeys = p + 1 - lo, per = (nkeys + nsplit - 1) / nsplit;
+  const int j0 = lo + z * per, j1 = min(p + 1, j0 + per);
   const T* kbase = kc + ((size_t)slot * max_len) * ldk + kh * dk;
-  const T* vbase = vc + ((size_t)slot * max_len) * ldv;
+  const T* vbase = vc + ((size_t)slot * max_len) * ldv + (GQA ? kh * dv : 0);
   float acc[MAXC];
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) acc[c] = 0.f;
@@ -42,8 +59,10 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
       float a = 0.f;
       for (int i = 0; i < dk; ++i) a += sq[i] * (float)kr[i];
       sc = a * scale;
+      if (GQA && x.bias != nullptr) sc += x.bias[(size_t)g * x.nd + min(p - j, x.nd - 1)];
     }
     const float mn = fmaxf(m, wave_max(sc));
+    if (mn == -INFINITY) continue;            // a split without keys (lanes agree: mn is wave-uniform)
     const float corr = expf(m - mn);          // m = -inf on the first chunk: exp(-inf) = 0
     const float w = j < j1 ? expf(sc - mn) : 0.f;
     l = l * corr + wave_sum(w);
@@ -93,27 +112,32 @@ __device__ __forceinline__ bf16x4 tr_read(const bf16* p) {
 
 // NW = 4 puts four query heads of one kv head (and one value head c) into a block: the key and value tiles are loaded
 // once into LDS for the four waves instead of once per head.
-template <int NDS, int NDT, bool HEADS, int NW>
+template <int NDS, int NDT, bool HEADS, int NW, bool GQA>
 __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restrict__ q, int ldq, const bf16* __restrict__ kc,
                                                        const bf16* __restrict__ vc, float* __restrict__ pm,
                                                        float* __restrict__ pl, float* __restrict__ pu,
                                                        const int* __restrict__ tile_seq, const int* __restrict__ tile_t0,
                                                        int H, int G, int dk, int dv, int ldk, int ldv, int max_len,
-                                                       int nsplit, float scale, SeqDesc d) {
+                                                       int nsplit, float scale, SeqDesc d, GqaExtra x) {
   constexpr int LDMAX = NDT * 32 + 8, LDKMAX = NDS * 16 + 8;
   __shared__ __attribute__((aligned(16))) bf16 sV[32 * LDMAX];
   __shared__ __attribute__((aligned(16))) bf16 sK[NW > 1 ? 32 * LDKMAX : 8];
-  const int tile = blockIdx.x, c = blockIdx.z % G, z = blockIdx.z / G;
+  const int tile = blockIdx.x, z = GQA ? blockIdx.z : blockIdx.z / G;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, hi = lane >> 5, ql = lane & 31, rep = H / G;
   const int s = tile_seq[tile], t0 = tile_t0[tile], tend = d.seq_off[s + 1], slot = d.slots[s];
   const int tq = HEADS ? t0 : min(t0 + ql, tend - 1);
   const int g = HEADS ? blockIdx.y * rep + min(ql, rep - 1) : blockIdx.y * NW + wv;
   const bool valid_q = HEADS ? ql < rep : t0 + ql < tend;
   const int pos_q = d.tok_pos[tq], pmax = HEADS ? pos_q : d.tok_pos[min(t0 + 31, tend - 1)];
-  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, LDK = dk + 8, GV = G * dv, kh = HEADS ? blockIdx.y : g / rep;
+  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, LDK = dk + 8, kh = HEADS ? blockIdx.y : g / rep;
+  const int c = GQA ? kh : blockIdx.z % G, GV = GQA ? dv : G * dv;
+  // block mask: the tile's sweep starts at the block of its first query; every query keeps its own block's keys
+  const int blk = GQA ? x.block : 0;
+  const int lo_t = blk > 0 ? ((HEADS ? pos_q : d.tok_pos[t0]) / blk) * blk : 0, lo_q = blk > 0 ? (pos_q / blk) * blk : 0;
+  const float* brow = (GQA && x.bias != nullptr) ? x.bias + (size_t)g * x.nd : nullptr;
   const float sl2 = scale * 1.4426950408889634f;   // scores in units of log2: v_exp_f32 is 2^x
   const int trow = 4 * (lane >> 5) + ((lane & 15) >> 2), tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-  const int per = (pmax + nsplit) / nsplit, j0 = z * per, j1 = min(pmax + 1, j0 + per);
+  const int per = (pmax - lo_t + nsplit) / nsplit, j0 = lo_t + z * per, j1 = min(pmax + 1, j0 + per);
   const bf16* kbase = kc + ((size_t)slot * max_len) * ldk + kh * dk + 8 * hi;
   const bf16* vbase = vc + ((size_t)slot * max_len) * ldv + c * dv;
   bf16x8 qf[NDS];
@@ -179,7 +203,10 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int key = jb + (r & 3) + 8 * (r >> 2) + 4 * hi;
-      sc[r] = (key <= pos_q && key < j1) ? sc[r] * sl2 : -INFINITY;
+      const bool seen = key <= pos_q && key < j1 && (!GQA || key >= lo_q);
+      float v = sc[r] * sl2;
+      if (GQA && brow != nullptr && seen) v += brow[min(pos_q - key, x.nd - 1)] * 1.4426950408889634f;
+      sc[r] = seen ? v : -INFINITY;
       mt = fmaxf(mt, sc[r]);
     }
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
@@ -217,8 +244,23 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
     }
   }
   if (!valid_q) return;
+  if (GQA && nsplit == 1) {                      // the whole softmax is here: add the sink, normalise, write
+    const float sk = x.sink_logit * 1.4426950408889634f, mf = x.sink ? fmaxf(m, sk) : m;
+    const float e = mf == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mf);
+    const float den = l * e + (x.sink ? __builtin_amdgcn_exp2f(sk - mf) : 0.f), inv = den > 0.f ? e / den : 0.f;
+    bf16* orow = (bf16*)x.out + (size_t)tq * (H * dv) + g * dv;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt < ndt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+          *reinterpret_cast<bf16x4*>(orow + dt * 32 + 8 * r4 + 4 * hi) =
+              bf16x4{(bf16)(acc[dt][4 * r4] * inv), (bf16)(acc[dt][4 * r4 + 1] * inv), (bf16)(acc[dt][4 * r4 + 2] * inv),
+                     (bf16)(acc[dt][4 * r4 + 3] * inv)};
+    return;
+  }
   const size_t o = ((size_t)tq * H + g) * nsplit + z;
-  if (c == 0 && hi == 0) {
+  if ((GQA || c == 0) && hi == 0) {
     pm[o] = m * 0.6931471805599453f;             // back to natural units, as the scalar sweep writes them
     pl[o] = l;
   }
@@ -227,7 +269,7 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
     if (dt < ndt)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4)
-        *reinterpret_cast<f32x4*>(pu + o * GV + c * dv + dt * 32 + 8 * r4 + 4 * hi) =
+        *reinterpret_cast<f32x4*>(pu + o * GV + (GQA ? 0 : c * dv) + dt * 32 + 8 * r4 + 4 * hi) =
             f32x4{acc[dt][4 * r4], acc[dt][4 * r4 + 1], acc[dt][4 * r4 + 2], acc[dt][4 * r4 + 3]};
 }
 
@@ -280,21 +322,20 @@ bool seq_attn_mfma_ok(int code, int ldq, int dk, int dv) {
   return code == 0 && dk % 16 == 0 && dk <= 256 && dv % 32 == 0 && dv <= 256 && ldq % 8 == 0;
 }
 
-// Pass 1 for any caller: the partial sweeps over a slot-indexed cache whose key rows are ldk and value rows ldv
-// elements apart (values may be columns of the key rows: a latent cache).  Writes pm, pl [T, H, nsplit] and
-// pu [T, H, nsplit, G * dv].
-void seq_attn_sweep(int code, const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, float* pm,
-                    float* pl, float* pu, int H, int G, int dk, int dv, int max_len, int nsplit, float scale,
-                    const int* tile_seq, const int* tile_t0, int ntiles, SeqDesc d, hipStream_t st) {
-  if (d.Ttot == 0) return;
+// Launches a sweep; returns true when it wrote the final output itself (GQA, matrix cores, one key split).
+template <bool GQA>
+static bool sweep(int code, const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, float* pm, float* pl,
+                  float* pu, int H, int G, int dk, int dv, int max_len, int nsplit, float scale, const int* tile_seq,
+                  const int* tile_t0, int ntiles, SeqDesc d, GqaExtra x, hipStream_t st) {
+  if (d.Ttot == 0) return false;
   if (tile_seq != nullptr && seq_attn_mfma_ok(code, ldq, dk, dv) && ldk % 8 == 0 && ldv % 8 == 0) {
     const bool heads = ntiles == d.Ttot && H / G <= 32 && H / G > 1;    // one token per tile: group the heads instead
     const int nw = (!heads && (H / G) % 4 == 0) ? 4 : 1;                 // four heads of a kv head share its tiles
-    const dim3 grid(ntiles, heads ? G : H / nw, G * nsplit);
+    const dim3 grid(ntiles, heads ? G : H / nw, GQA ? nsplit : G * nsplit);
 #define SEQ_ATTN_LAUNCH(NDS, NDT, HEADS, NW)                                                                        \
-  hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS, NW>), grid, dim3(64 * NW), 0, st, (const bf16*)q, ldq,       \
+  hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS, NW, GQA>), grid, dim3(64 * NW), 0, st, (const bf16*)q, ldq,  \
                      (const bf16*)kc, (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, ldk, ldv, max_len, \
-                     nsplit, scale, d)
+                     nsplit, scale, d, x)
     if (dk <= 128 && dv <= 128) {
       if (heads) SEQ_ATTN_LAUNCH(8, 4, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(8, 4, false, 4); else SEQ_ATTN_LAUNCH(8, 4, false, 1);
     } else {
@@ -302,12 +343,58 @@ void seq_attn_sweep(int code, const void* q, int ldq, const void* kc, int ldk, c
     }
 #undef SEQ_ATTN_LAUNCH
     LIPA_CHECK_LAUNCH();
-    return;
+    return GQA && nsplit == 1;
   }
   SEQ_DISPATCH_T(code, {
-    hipLaunchKernelGGL(k_talk_attn_partial<T>, dim3(d.Ttot, H, nsplit), dim3(64), sizeof(float) * dk, st, (const T*)q,
-                       ldq, (const T*)kc, (const T*)vc, pm, pl, pu, H, G, dk, dv, ldk, ldv, max_len, nsplit, scale, d);
+    hipLaunchKernelGGL((k_talk_attn_partial<T, GQA>), dim3(d.Ttot, H, nsplit), dim3(64), sizeof(float) * dk, st,
+                       (const T*)q, ldq, (const T*)kc, (const T*)vc, pm, pl, pu, H, G, dk, dv, ldk, ldv, max_len, nsplit,
+                       scale, d, x);
   });
+  LIPA_CHECK_LAUNCH();
+  return false;
+}
+
+// Pass 1 for any caller: the partial sweeps over a slot-indexed cache whose key rows are ldk and value rows ldv
+// elements apart (values may be columns of the key rows: a latent cache).  Writes pm, pl [T, H, nsplit] and
+// pu [T, H, nsplit, G * dv].
+void seq_attn_sweep(int code, const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, float* pm,
+                    float* pl, float* pu, int H, int G, int dk, int dv, int max_len, int nsplit, float scale,
+                    const int* tile_seq, const int* tile_t0, int ntiles, SeqDesc d, hipStream_t st) {
+  sweep<false>(code, q, ldq, kc, ldk, vc, ldv, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale, tile_seq, tile_t0,
+               ntiles, d, GqaExtra{nullptr, 0, 0, 0, 0.f, nullptr}, st);
+}
+
+// Merge of a GQA sweep's key splits: one wave per (token, head); the sink joins the denominator here.
+template <typename T>
+__global__ __launch_bounds__(64) void k_gqa_merge(const float* __restrict__ pm, const float* __restrict__ pl,
+                                                  const float* __restrict__ pu, T* __restrict__ out, int H, int dv,
+                                                  int nsplit, int sink, float sink_logit) {
+  const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  const size_t b = ((size_t)t * H + g) * nsplit;
+  float mx = sink ? sink_logit : -INFINITY;
+  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pm[b + z]);
+  float l = sink ? expf(sink_logit - mx) : 0.f;
+  for (int z = 0; z < nsplit; ++z) l += pm[b + z] == -INFINITY ? 0.f : expf(pm[b + z] - mx) * pl[b + z];
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int col = lane; col < dv; col += 64) {
+    float u = 0.f;
+    for (int z = 0; z < nsplit; ++z)
+      if (pm[b + z] != -INFINITY) u += expf(pm[b + z] - mx) * pu[(b + z) * dv + col];
+    out[(size_t)t * (H * dv) + g * dv + col] = (T)(u * inv);
+  }
+}
+
+// Grouped-query attention over a slot-indexed cache with an optional distance bias, block mask and sink.
+void seq_gqa_attention(int code, const void* q, int ldq, const void* kc, const void* vc, float* pm, float* pl, float* pu,
+                       const float* bias, int nd, int block, int sink, float sink_logit, void* out, int H, int G, int dk,
+                       int dv, int max_len, int nsplit, float scale, const int* tile_seq, const int* tile_t0, int ntiles,
+                       SeqDesc d, hipStream_t st) {
+  if (d.Ttot == 0) return;
+  const bool direct = sweep<true>(code, q, ldq, kc, G * dk, vc, G * dv, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale,
+                                  tile_seq, tile_t0, ntiles, d, GqaExtra{bias, nd, block, sink, sink_logit, out}, st);
+  if (direct) return;
+  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_gqa_merge<T>, dim3(d.Ttot, H), dim3(64), 0, st, pm, pl, pu, (T*)out, H, dv,
+                                          nsplit, sink, sink_logit));
   LIPA_CHECK_LAUNCH();
 }
 

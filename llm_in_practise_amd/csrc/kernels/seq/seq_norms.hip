@@ -279,6 +279,106 @@ __global__ __launch_bounds__(256) void k_gate_group_norm(const float* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------- launchers
+// x[t, s, c] = table[tok[t], c] + ptable[pos[t], c] for every stream s (learned positions, not scaled); a position past
+// the table reads its last row (rows nobody reads may carry any position)
+template <typename T>
+__global__ __launch_bounds__(256) void k_embed_learned(const long* __restrict__ tok, const int* __restrict__ pos,
+                                                       const T* __restrict__ table, const T* __restrict__ ptable,
+                                                       float* __restrict__ x, int W, int S, int prow, int vocab) {
+  const size_t t = blockIdx.x;
+  const size_t id = (size_t)min(max(tok[t], 0l), (long)vocab - 1), p = (size_t)min(max(pos[t], 0), prow - 1);
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = (float)table[id * W + c] + (float)ptable[p * W + c];
+    for (int s = 0; s < S; ++s) x[(t * S + s) * W + c] = v;
+  }
+}
+
+// Several residual streams X [T, S, W] (float, in place).  With a sublayer output y: X_t <- sum_s mix[s, t] X_s +
+// out[t] y for all t at once; then h = rmsnorm(sum_s read[s] X_s) * w, the next sublayer's input.  y == null: only h.
+constexpr int MAXS = 8;
+template <typename T, typename YT>
+__global__ __launch_bounds__(256) void k_hyper_mix_norm(float* __restrict__ X, const YT* __restrict__ y, int ldy,
+                                                        const float* __restrict__ mix, const float* __restrict__ outw,
+                                                        const float* __restrict__ read, const float* __restrict__ w,
+                                                        T* __restrict__ h, int W, int S, float eps) {
+  __shared__ float sc[4];
+  __shared__ float sm[MAXS * MAXS + 2 * MAXS];
+  const size_t t = blockIdx.x;
+  float* smix = sm;
+  float* sout = sm + MAXS * MAXS;
+  float* srd = sout + MAXS;
+  if (threadIdx.x < S * S) smix[threadIdx.x] = y != nullptr ? mix[threadIdx.x] : 0.f;
+  if (threadIdx.x < S) {
+    sout[threadIdx.x] = y != nullptr ? outw[threadIdx.x] : 0.f;
+    srd[threadIdx.x] = read[threadIdx.x];
+  }
+  __syncthreads();
+  float* xr = X + t * S * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float old[MAXS], u = 0.f;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) old[s] = s < S ? xr[(size_t)s * W + c] : 0.f;
+    if (y != nullptr) {
+      const float yv = (float)y[t * ldy + c];
+#pragma unroll
+      for (int k = 0; k < MAXS; ++k)
+        if (k < S) {
+          float v = sout[k] * yv;
+#pragma unroll
+          for (int s = 0; s < MAXS; ++s)
+            if (s < S) v += smix[s * S + k] * old[s];
+          xr[(size_t)k * W + c] = v;
+          u += srd[k] * v;
+        }
+    } else {
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s)
+        if (s < S) u += srd[s] * old[s];
+    }
+    ss += u * u;
+  }
+  const float rs = rsqrtf(block_sum256(ss, sc) / W + eps);
+  for (int c = threadIdx.x; c < W; c += 256) {      // the thread re-reads the columns it wrote itself
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s)
+      if (s < S) u += srd[s] * xr[(size_t)s * W + c];
+    h[t * W + c] = (T)(u * rs * w[c]);
+  }
+}
+
+// A step's [q | k | v] rows on their way into attention: q and k RMS-normed over their whole width, the normed k and
+// the values (blended with another cache's values of the same slot and position when vfirst is given:
+// (1 - lam) v + lam vfirst) written to the slot cache rows of each token's position.
+template <typename T>
+__global__ __launch_bounds__(256) void k_qk_norm_store(const T* __restrict__ u, int ldu, const float* __restrict__ qw,
+                                                       const float* __restrict__ kw, T* __restrict__ qout,
+                                                       T* __restrict__ kc, T* __restrict__ vc,
+                                                       const T* __restrict__ vfirst, const float* __restrict__ lam,
+                                                       int nq, int nk, int nv, int max_len, float eps, SeqDesc d) {
+  __shared__ float sc[4];
+  const size_t t = blockIdx.x;
+  const T* r = u + t * ldu;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x; c < nq; c += 256) { const float v = (float)r[c]; sq += v * v; }
+  for (int c = threadIdx.x; c < nk; c += 256) { const float v = (float)r[nq + c]; sk += v * v; }
+  const float rq = rsqrtf(block_sum256(sq, sc) / nq + eps);
+  const float rk = rsqrtf(block_sum256(sk, sc) / nk + eps);
+  for (int c = threadIdx.x; c < nq; c += 256) qout[t * nq + c] = (T)((float)r[c] * rq * qw[c]);
+  const int pos = d.tok_pos[t], slot = d.slots[d.tok_seq[t]];
+  if (pos < 0 || pos >= max_len) return;             // a row nobody reads may carry any position
+  const size_t row = (size_t)slot * max_len + pos;
+  for (int c = threadIdx.x; c < nk; c += 256) kc[row * nk + c] = (T)((float)r[nq + c] * rk * kw[c]);
+  if (vfirst != nullptr) {
+    const float l = lam[0];
+    for (int c = threadIdx.x; c < nv; c += 256)
+      vc[row * nv + c] = (T)((1.f - l) * (float)r[nq + nk + c] + l * (float)vfirst[row * nv + c]);
+  } else {
+    for (int c = threadIdx.x; c < nv; c += 256) vc[row * nv + c] = r[nq + nk + c];
+  }
+}
+
 void seq_embed_sincos(int code, const long* tok, const int* pos, const void* table, const float* inv_freq, float* x,
                       int T_, int W, float scale, hipStream_t st) {
   if (T_ == 0) return;
@@ -375,5 +475,38 @@ void seq_gate_group_norm(int code, const float* y, const void* z, int ldz, const
       hipLaunchKernelGGL((k_gate_group_norm<T, false>), dim3(T_, parts), dim3(256), 0, st, y, (const T*)z, ldz, w,
                          (T*)out, n, gs, eps);
   });
+  LIPA_CHECK_LAUNCH();
+}
+
+int seq_hyper_max_streams() { return MAXS; }
+
+void seq_embed_learned(int code, const long* tok, const int* pos, const void* table, const void* ptable, float* x, int T_,
+                       int W, int S, int prow, int vocab, hipStream_t st) {
+  if (T_ == 0) return;
+  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_embed_learned<T>, dim3(T_), dim3(256), 0, st, tok, pos, (const T*)table,
+                                          (const T*)ptable, x, W, S, prow, vocab));
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_hyper_mix_norm(int code, int y_f32, float* X, const void* y, int ldy, const float* mix, const float* outw,
+                        const float* read, const float* w, void* h, int T_, int W, int S, float eps, hipStream_t st) {
+  if (T_ == 0) return;
+  SEQ_DISPATCH_T(code, {
+    if (y_f32)
+      hipLaunchKernelGGL((k_hyper_mix_norm<T, float>), dim3(T_), dim3(256), 0, st, X, (const float*)y, ldy, mix, outw,
+                         read, w, (T*)h, W, S, eps);
+    else
+      hipLaunchKernelGGL((k_hyper_mix_norm<T, T>), dim3(T_), dim3(256), 0, st, X, (const T*)y, ldy, mix, outw, read, w,
+                         (T*)h, W, S, eps);
+  });
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_qk_norm_store(int code, const void* u, int ldu, const float* qw, const float* kw, void* qout, void* kc, void* vc,
+                       const void* vfirst, const float* lam, int nq, int nk, int nv, int max_len, float eps, SeqDesc d,
+                       hipStream_t st) {
+  if (d.Ttot == 0) return;
+  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_qk_norm_store<T>, dim3(d.Ttot), dim3(256), 0, st, (const T*)u, ldu, qw, kw,
+                                          (T*)qout, (T*)kc, (T*)vc, (const T*)vfirst, lam, nq, nk, nv, max_len, eps, d));
   LIPA_CHECK_LAUNCH();
 }

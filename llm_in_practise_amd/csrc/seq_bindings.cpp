@@ -46,13 +46,24 @@ void seq_latent_q_assemble(int, const void*, size_t, size_t, const void*, int, i
                            int, SeqDesc, hipStream_t);
 void seq_latent_merge(int, const float*, const float*, const float*, const void*, int, void*, int, int, int, int,
                       hipStream_t);
-void seq_route_grouped(const float*, const float*, int*, float*, int, int, int, int, int, float, hipStream_t);
+void seq_route_grouped(const float*, const float*, int*, float*, int, int, int, int, int, float, int, hipStream_t);
 void seq_route_fused(int, const void*, int, const float*, const float*, int*, float*, int, int, int, int, int, int, float,
-                     hipStream_t);
-void seq_moe_pairs(int, const void*, int, const void*, const void*, const int*, const float*, const void*, void*, float*,
-                   int, int, int, int, int, float, hipStream_t);
-void seq_moe_combine(int, const void*, const long*, const int*, const float*, const void*, int, const void*, float*, int,
-                     int, int, int, hipStream_t);
+                     int, int, float*, hipStream_t);
+void seq_moe_pairs(int, const void*, int, const void*, const void*, const int*, const float*, const void*, const float*,
+                   void*, float*, int, int, int, int, int, float, int, hipStream_t);
+void seq_moe_combine(int, const void*, const long*, const int*, const float*, const void*, int, const void*, const float*,
+                     float*, int, int, int, int, hipStream_t);
+void seq_embed_learned(int, const long*, const int*, const void*, const void*, float*, int, int, int, int, int,
+                       hipStream_t);
+void seq_hyper_mix_norm(int, int, float*, const void*, int, const float*, const float*, const float*, const float*, void*,
+                        int, int, int, float, hipStream_t);
+void seq_qk_norm_store(int, const void*, int, const float*, const float*, void*, void*, void*, const void*, const float*,
+                       int, int, int, int, float, SeqDesc, hipStream_t);
+void seq_gqa_attention(int, const void*, int, const void*, const void*, float*, float*, float*, const float*, int, int,
+                       int, float, void*, int, int, int, int, int, int, float, const int*, const int*, int, SeqDesc,
+                       hipStream_t);
+int seq_hyper_max_streams();
+bool seq_attn_mfma_ok(int, int, int, int);
 void seq_ff_act(int, const void*, void*, int, int, int, float, hipStream_t);
 int seq_route_max_outputs();
 void seq_mlstm_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, const float*,
@@ -542,7 +553,7 @@ Tensor latent_attention(Tensor qa, Tensor q, Tensor cache, optional<Tensor> gate
 // ---- mixture of experts
 static const float* check_routing(int64_t n, const optional<Tensor>& corr, int64_t top, int64_t groups, int64_t keep) {
   TORCH_CHECK(n >= 1 && n <= seq_route_max_outputs(), "router outputs above ", seq_route_max_outputs());
-  TORCH_CHECK(top >= 1 && top <= n, "top");
+  TORCH_CHECK(top >= 1 && top <= n && top <= 64, "top");
   TORCH_CHECK(groups >= 1 && groups <= 64 && n % groups == 0 && keep >= 1 && keep <= groups, "groups must divide n");
   TORCH_CHECK(top <= keep * (n / groups), "fewer eligible outputs than `top`");
   if (corr && corr->defined()) {
@@ -554,7 +565,8 @@ static const float* check_routing(int64_t n, const optional<Tensor>& corr, int64
 }
 
 std::vector<Tensor> route_grouped(Tensor z, optional<Tensor> corr, int64_t top, int64_t groups, int64_t keep,
-                                  double scale) {
+                                  double scale, int64_t kind) {
+  TORCH_CHECK(kind >= 0 && kind < 8, "routing kind");
   f32c(z, "router logits");
   TORCH_CHECK(z.dim() == 2, "router logits: [T, n]");
   const int64_t T = z.size(0), n = z.size(1);
@@ -562,13 +574,15 @@ std::vector<Tensor> route_grouped(Tensor z, optional<Tensor> corr, int64_t top, 
   auto idx = at::empty({T, top}, z.options().dtype(at::kInt));
   auto w = at::empty({T, top}, z.options());
   seq_route_grouped(z.data_ptr<float>(), cp, idx.data_ptr<int>(), w.data_ptr<float>(), (int)T, (int)n, (int)top,
-                    (int)groups, (int)keep, (float)scale, stream());
+                    (int)groups, (int)keep, (float)scale, (int)kind, stream());
   return {idx, w};
 }
 
 // the router product (float weights [n, W], activations h [T, W] as they are, float accumulation) and the routing
+// the last `extra` router rows are not routed: their products come back as a third tensor, float [T, extra]
 std::vector<Tensor> route_fused(Tensor h, Tensor router, optional<Tensor> corr, int64_t top, int64_t groups,
-                                int64_t keep, double scale) {
+                                int64_t keep, double scale, int64_t kind, int64_t extra) {
+  TORCH_CHECK(kind >= 0 && kind < 8, "routing kind");
   const int code = code_of(h);
   TORCH_CHECK(h.dim() == 2, "h: [T, W]");
   const int64_t T = h.size(0), W = h.size(1);
@@ -576,12 +590,15 @@ std::vector<Tensor> route_fused(Tensor h, Tensor router, optional<Tensor> corr, 
   f32c(router, "router");
   TORCH_CHECK(router.dim() == 2 && router.size(1) == W, "router: [n, W]");
   const int64_t n = router.size(0);
-  const float* cp = check_routing(n, corr, top, groups, keep);
+  TORCH_CHECK(extra >= 0 && extra < n && n <= seq_route_max_outputs(), "router rows");
+  const float* cp = check_routing(n - extra, corr, top, groups, keep);
   auto idx = at::empty({T, top}, h.options().dtype(at::kInt));
   auto w = at::empty({T, top}, h.options().dtype(at::kFloat));
+  auto ex = at::empty({T, extra}, h.options().dtype(at::kFloat));
   seq_route_fused(code, h.data_ptr(), ld(h), router.data_ptr<float>(), cp, idx.data_ptr<int>(), w.data_ptr<float>(),
-                  (int)T, (int)n, (int)W, (int)top, (int)groups, (int)keep, (float)scale, stream());
-  return {idx, w};
+                  (int)T, (int)n, (int)W, (int)top, (int)groups, (int)keep, (float)scale, (int)kind, (int)extra,
+                  ex.data_ptr<float>(), stream());
+  return {idx, w, ex};
 }
 
 static void check_route(const Tensor& idx, const Tensor& w, int64_t T) {
@@ -592,7 +609,16 @@ static void check_route(const Tensor& idx, const Tensor& w, int64_t T) {
 }
 
 // few tokens: every (token, expert) pair streams its expert.  wgu [E, 2, F, W], wd [E, W, F]; returns float [T, W]
-Tensor moe_pairs(Tensor h, Tensor wgu, Tensor wd, Tensor idx, Tensor w, optional<Tensor> shared, double limit) {
+static const float* shared_gate_of(const optional<Tensor>& sg, int64_t T) {
+  if (!(sg && sg->defined())) return nullptr;
+  f32c(*sg, "shared gate");
+  TORCH_CHECK(sg->numel() == T, "shared gate: float [T]");
+  return sg->data_ptr<float>();
+}
+
+Tensor moe_pairs(Tensor h, Tensor wgu, Tensor wd, Tensor idx, Tensor w, optional<Tensor> shared, double limit,
+                 int64_t mode, optional<Tensor> shared_gate) {
+  TORCH_CHECK(mode == 1 || mode == 2, "expert activation: 1 clipped GLU, 2 SiLU GLU");
   const int code = code_of(h);
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous(), "h: [T, W] contiguous");
   const int64_t T = h.size(0), W = h.size(1);
@@ -613,12 +639,14 @@ Tensor moe_pairs(Tensor h, Tensor wgu, Tensor wd, Tensor idx, Tensor w, optional
   auto a = at::empty({T * top, F}, h.options());
   auto out = at::empty({T, W}, h.options().dtype(at::kFloat));
   seq_moe_pairs(code, h.data_ptr(), (int)W, wgu.data_ptr(), wd.data_ptr(), idx.data_ptr<int>(), w.data_ptr<float>(), sp,
-                a.data_ptr(), out.data_ptr<float>(), (int)T, (int)top, (int)E, (int)F, (int)W, (float)limit, stream());
+                shared_gate_of(shared_gate, T), a.data_ptr(), out.data_ptr<float>(), (int)T, (int)top, (int)E, (int)F,
+                (int)W, (float)limit, (int)mode, stream());
   return out;
 }
 
 // ys [rows, W]: expert outputs in expert-sorted order; pos [T, top] int64: the row of every pair
-Tensor moe_combine_sorted(Tensor ys, Tensor pos, Tensor idx, Tensor w, Tensor h, optional<Tensor> shared, int64_t E) {
+Tensor moe_combine_sorted(Tensor ys, Tensor pos, Tensor idx, Tensor w, Tensor h, optional<Tensor> shared, int64_t E,
+                          optional<Tensor> shared_gate) {
   const int code = code_of(h);
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous(), "h: [T, W] contiguous");
   const int64_t T = h.size(0), W = h.size(1);
@@ -634,16 +662,151 @@ Tensor moe_combine_sorted(Tensor ys, Tensor pos, Tensor idx, Tensor w, Tensor h,
   }
   auto out = at::empty({T, W}, h.options().dtype(at::kFloat));
   seq_moe_combine(code, ys.data_ptr(), pos.data_ptr<long>(), idx.data_ptr<int>(), w.data_ptr<float>(), h.data_ptr(),
-                  (int)W, sp, out.data_ptr<float>(), (int)T, (int)idx.size(1), (int)E, (int)W, stream());
+                  (int)W, sp, shared_gate_of(shared_gate, T), out.data_ptr<float>(), (int)T, (int)idx.size(1), (int)E,
+                  (int)W, stream());
   return out;
 }
 
-// mode 0: tanh-form GELU of z [T, F]; mode 1: clipped GLU of z [T, 2F] = [gate | up]
+// mode 0: tanh-form GELU of z [T, F]; mode 1: clipped GLU, mode 2: SiLU GLU of z [T, 2F] = [gate | up]
 Tensor ff_act(Tensor z, int64_t mode, double limit) {
-  TORCH_CHECK(z.is_cuda() && z.is_contiguous() && z.dim() == 2 && (mode == 0 || (mode == 1 && z.size(1) % 2 == 0)), "z");
+  TORCH_CHECK(z.is_cuda() && z.is_contiguous() && z.dim() == 2 &&
+                  (mode == 0 || ((mode == 1 || mode == 2) && z.size(1) % 2 == 0)), "z");
   const int64_t T = z.size(0), F = mode == 0 ? z.size(1) : z.size(1) / 2;
   auto out = at::empty({T, F}, z.options());
   seq_ff_act(code_of(z), z.data_ptr(), out.data_ptr(), (int)T, (int)F, (int)mode, (float)limit, stream());
+  return out;
+}
+
+// ---- learned positions, several residual streams, q/k norm + cache write, biased block attention with a sink
+Tensor embed_learned(Tensor tok, Tensor pos, Tensor table, Tensor ptable, int64_t streams) {
+  TORCH_CHECK(tok.is_cuda() && tok.scalar_type() == at::kLong && tok.is_contiguous(), "tokens: int64");
+  TORCH_CHECK(pos.is_cuda() && pos.scalar_type() == at::kInt && pos.is_contiguous() && pos.numel() == tok.numel(),
+              "positions: int32, one per token");
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2 && ptable.is_cuda() && ptable.is_contiguous() &&
+                  ptable.dim() == 2 && ptable.size(1) == table.size(1) && ptable.scalar_type() == table.scalar_type() &&
+                  ptable.size(0) >= 1 && table.size(0) >= 1, "token and position tables: [rows, W], one dtype");
+  TORCH_CHECK(streams >= 1 && streams <= seq_hyper_max_streams(), "streams: 1..", seq_hyper_max_streams());
+  const int T = (int)tok.numel(), W = (int)table.size(1);
+  auto x = at::empty({T, streams, W}, table.options().dtype(at::kFloat));
+  seq_embed_learned(code_of(table), tok.data_ptr<long>(), pos.data_ptr<int>(), table.data_ptr(), ptable.data_ptr(),
+                    x.data_ptr<float>(), T, W, (int)streams, (int)ptable.size(0), (int)table.size(0), stream());
+  return x;
+}
+
+// X float [T, S, W] in place; y [T, W] (activation dtype or float) or none; returns the next sublayer's input [T, W]
+Tensor hyper_mix_norm(Tensor X, optional<Tensor> y, optional<Tensor> mix, optional<Tensor> outw, Tensor read, Tensor w,
+                      double eps, bool out_bf16) {
+  f32c(X, "streams");
+  TORCH_CHECK(X.dim() == 3, "streams: [T, S, W]");
+  const int64_t T = X.size(0), S = X.size(1), W = X.size(2);
+  TORCH_CHECK(S >= 1 && S <= seq_hyper_max_streams(), "streams: 1..", seq_hyper_max_streams());
+  f32c(read, "read weights");
+  f32c(w, "norm weight");
+  TORCH_CHECK(read.numel() == S && w.numel() == W, "read weights [S], norm weight [W]");
+  const void* yp = nullptr;
+  const float* mp = nullptr;
+  const float* op = nullptr;
+  int ldy = 0, y_f32 = 0;
+  if (y && y->defined()) {
+    TORCH_CHECK(mix && mix->defined() && outw && outw->defined(), "a sublayer output needs mix and out weights");
+    f32c(*mix, "mix");
+    f32c(*outw, "out weights");
+    TORCH_CHECK(mix->numel() == S * S && outw->numel() == S, "mix [S, S], out weights [S]");
+    y_f32 = y->scalar_type() == at::kFloat;
+    rows(*y, T, W, code_of(*y), "y");
+    TORCH_CHECK(y_f32 || !out_bf16 || y->scalar_type() == at::kBFloat16, "y: float or the activation dtype");
+    TORCH_CHECK(y_f32 || (code_of(*y) == (out_bf16 ? 0 : 1)), "y: float or the activation dtype");
+    yp = y->data_ptr();
+    ldy = ld(*y);
+    mp = mix->data_ptr<float>();
+    op = outw->data_ptr<float>();
+  }
+  auto h = at::empty({T, W}, X.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
+  seq_hyper_mix_norm(out_bf16 ? 0 : 1, y_f32, X.data_ptr<float>(), yp, ldy, mp, op, read.data_ptr<float>(),
+                     w.data_ptr<float>(), h.data_ptr(), (int)T, (int)W, (int)S, (float)eps, stream());
+  return h;
+}
+
+static void check_kv_cache(const Tensor& c, int64_t cols, int code, const char* n) {
+  TORCH_CHECK(c.is_cuda() && c.is_contiguous() && c.dim() == 3 && c.size(2) == cols && code_of(c) == code, n,
+              ": [slots, max_len, columns] in the activation dtype");
+}
+
+// u [T, nq + nk + nv]; returns the normed q [T, nq]; k and v rows go to the caches at each token's (slot, position).
+// Slots are rows of the engine's pool (SeqBatch checks them on the host); the kernel skips positions outside the cache.
+Tensor qk_norm_store(Tensor u, int64_t nq, int64_t nk, Tensor qw, Tensor kw, Tensor kc, Tensor vc,
+                     optional<Tensor> vfirst, optional<Tensor> lam, double eps, std::vector<Tensor> desc) {
+  const int code = code_of(u);
+  TORCH_CHECK(u.dim() == 2 && nq >= 1 && nk >= 1 && u.size(1) > nq + nk, "u: [T, nq + nk + nv]");
+  const int64_t T = u.size(0), nv = u.size(1) - nq - nk;
+  rows(u, T, nq + nk + nv, code, "u");
+  f32c(qw, "q norm weight");
+  f32c(kw, "k norm weight");
+  TORCH_CHECK(qw.numel() == nq && kw.numel() == nk, "norm weights: [nq], [nk]");
+  check_kv_cache(kc, nk, code, "key cache");
+  check_kv_cache(vc, nv, code, "value cache");
+  TORCH_CHECK(vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "caches: one pool of slots");
+  const void* fp = nullptr;
+  const float* lp = nullptr;
+  if (vfirst && vfirst->defined()) {
+    check_kv_cache(*vfirst, nv, code, "first value cache");
+    TORCH_CHECK(vfirst->sizes() == vc.sizes() && lam && lam->defined(), "first value cache: the value cache's shape");
+    f32c(*lam, "lambda");
+    TORCH_CHECK(lam->numel() == 1, "lambda: one float");
+    fp = vfirst->data_ptr();
+    lp = lam->data_ptr<float>();
+  }
+  SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  auto q = at::empty({T, nq}, u.options());
+  seq_qk_norm_store(code, u.data_ptr(), ld(u), qw.data_ptr<float>(), kw.data_ptr<float>(), q.data_ptr(), kc.data_ptr(),
+                    vc.data_ptr(), fp, lp, (int)nq, (int)nk, (int)nv, (int)kc.size(1), (float)eps, d, stream());
+  return q;
+}
+
+Tensor biased_attention(Tensor q, Tensor kc, Tensor vc, optional<Tensor> bias, int64_t H, int64_t G, double scale,
+                        int64_t block, bool sink, double sink_logit, int64_t nsplit, std::vector<Tensor> desc,
+                        std::vector<Tensor> tiles) {
+  const int code = code_of(q);
+  TORCH_CHECK(q.dim() == 2 && H >= 1 && G >= 1 && H % G == 0 && q.size(1) % H == 0, "q: [T, H * dk]");
+  const int64_t T = q.size(0), dk = q.size(1) / H;
+  rows(q, T, H * dk, code, "q");
+  check_kv_cache(kc, G * dk, code, "key cache");
+  TORCH_CHECK(vc.is_cuda() && vc.is_contiguous() && vc.dim() == 3 && vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1) &&
+                  vc.size(2) % G == 0 && code_of(vc) == code, "value cache: [slots, max_len, G * dv]");
+  const int64_t dv = vc.size(2) / G, max_len = kc.size(1);
+  TORCH_CHECK(dv >= 1 && dv <= seq_attn_max_cols(), "attention: dv above ", seq_attn_max_cols());
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 1024 && block >= 0, "nsplit, block");
+  const float* bp = nullptr;
+  int nd = 0;
+  if (bias && bias->defined()) {
+    f32c(*bias, "distance bias");
+    TORCH_CHECK(bias->dim() == 2 && bias->size(0) == H && bias->size(1) >= 1, "distance bias: [H, distances]");
+    bp = bias->data_ptr<float>();
+    nd = (int)bias->size(1);
+  }
+  SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  const int* tseq = nullptr;
+  const int* tt0 = nullptr;
+  int ntiles = 0;
+  if (tiles.size() == 2) {
+    for (auto& t : tiles) TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), "tiles: int32");
+    TORCH_CHECK(tiles[0].numel() == tiles[1].numel(), "tiles: two arrays of one length");
+    tseq = tiles[0].data_ptr<int>();
+    tt0 = tiles[1].data_ptr<int>();
+    ntiles = (int)tiles[0].numel();
+    TORCH_CHECK((int64_t)ntiles * 32 >= T && nsplit <= 65535 && H <= 65535, "tiles must cover the tokens");
+  }
+  auto fo = q.options().dtype(at::kFloat);
+  // one key split on the matrix-core sweep writes the output itself: no partial sums
+  const bool direct = nsplit == 1 && tseq != nullptr && seq_attn_mfma_ok(code, ld(q), (int)dk, (int)dv) &&
+                      (G * dk) % 8 == 0 && (G * dv) % 8 == 0;
+  const int64_t np = direct ? 0 : T;
+  auto pm = at::empty({np, H, nsplit}, fo), pl = at::empty({np, H, nsplit}, fo);
+  auto pu = at::empty({np, H, nsplit, dv}, fo);
+  auto out = at::empty({T, H * dv}, q.options());
+  seq_gqa_attention(code, q.data_ptr(), ld(q), kc.data_ptr(), vc.data_ptr(), pm.data_ptr<float>(), pl.data_ptr<float>(),
+                    pu.data_ptr<float>(), bp, nd, (int)block, sink ? 1 : 0, (float)sink_logit, out.data_ptr(), (int)H,
+                    (int)G, (int)dk, (int)dv, (int)max_len, (int)nsplit, (float)scale, tseq, tt0, ntiles, d, stream());
   return out;
 }
 
@@ -673,4 +836,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_pairs", &moe_pairs);
   m.def("moe_combine_sorted", &moe_combine_sorted);
   m.def("ff_act", &ff_act);
+  m.def("embed_learned", &embed_learned);
+  m.def("hyper_mix_norm", &hyper_mix_norm);
+  m.def("qk_norm_store", &qk_norm_store);
+  m.def("biased_attention", &biased_attention);
 }

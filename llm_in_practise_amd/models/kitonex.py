@@ -62,6 +62,7 @@ class KitonexConfig:
     @classmethod
     def from_dict(cls, d: dict) -> "KitonexConfig":
         layers = copy.deepcopy(d["layers"])
+        blended = set()
         for lc in layers:
             if lc["type"] != "attention":
                 raise ValueError(f"Kitonex: unknown layer type {lc['type']!r}")
@@ -71,6 +72,10 @@ class KitonexConfig:
             m = lc["mixer"]
             if int(m["heads"]) % int(m.get("kv_heads", m["heads"])):
                 raise ValueError("Kitonex: heads must be a multiple of kv_heads")
+            if m.get("v_mix"):
+                blended.add(int(m.get("kv_heads", m["heads"])) * int(m["vdim"]))
+        if len(blended) > 1:
+            raise ValueError("Kitonex: layers that blend values (v_mix) must have value rows of one width")
         return cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers,
                    norm_eps=float(d.get("norm", {}).get("eps", 1e-6)), streams=int(d.get("streams", 1)),
                    max_positions=int(d.get("max_positions", 2048)))
@@ -328,7 +333,7 @@ class KitonexModel(SeqStateModel):
     def run(self, tokens: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
         """Packed tokens ``[T]`` through all layers; returns the final-normed hidden states ``[T, width]``."""
         cfg, L, eps = self.cfg, self.layers, self.cfg.norm_eps
-        if sb.max_pos > self.pos_table.shape[0]:
+        if not sb.decode and sb.max_pos > self.pos_table.shape[0]:
             raise ValueError(f"Kitonex: a sequence passes the {self.pos_table.shape[0]} learned positions")
         X = embed_learned(tokens, sb.desc[4], self.embed_tokens, self.pos_table, cfg.streams)
         h = hyper_mix_norm(X, None, None, None, L[0].t.read1, L[0].t.norm1, eps, self.dtype)

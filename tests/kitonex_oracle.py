@@ -11,6 +11,7 @@ import math
 import torch
 
 F64 = torch.float64
+SINK = 1.0      # what every softmax denominator carries besides its keys (a test sets 0 to show that it matters)
 
 
 def rms(x, w, eps):
@@ -57,7 +58,7 @@ def sink_attention(q, k, v, rel, H, G, scale, chunk, far):
                 s[j - lo] = (q[i, h * dk:(h + 1) * dk] * k[j, g * dk:(g + 1) * dk]).sum() * scale \
                     + rel[distance_bucket(i - j, rel.shape[0], far), h]
             e = torch.exp(s)
-            p = e / (1.0 + e.sum())
+            p = e / (SINK + e.sum())
             out[i, h * dv:(h + 1) * dv] = (p[:, None] * v[lo:i + 1, g * dv:(g + 1) * dv]).sum(0)
     return out
 
@@ -75,13 +76,13 @@ def sink_attention_fast(q, k, v, rel, H, G, scale, chunk, far):
         g = h // (H // G)
         s = q[:, h * dk:(h + 1) * dk] @ k[:, g * dk:(g + 1) * dk].t() * scale + rel[:, h][bucket]
         e = torch.where(seen, torch.exp(s), torch.zeros((), dtype=F64))
-        out[:, h * dv:(h + 1) * dv] = (e / (1.0 + e.sum(-1, keepdim=True))) @ v[:, g * dv:(g + 1) * dv]
+        out[:, h * dv:(h + 1) * dv] = (e / (SINK + e.sum(-1, keepdim=True))) @ v[:, g * dv:(g + 1) * dv]
     return out
 
 
 def attention_mixer(m, W, p, h, eps, v_first, fast=True):
     """Returns (output, this layer's values before mixing or None)."""
-    H, G = m["heads"], m["kv_heads"]
+    H, G = m["heads"], m.get("kv_heads", m["heads"])
     proj = {}
     for n in "qkv":
         u = h @ W[p + n].to(F64).t() + W[p + n + ".b"].to(F64)
@@ -97,7 +98,8 @@ def attention_mixer(m, W, p, h, eps, v_first, fast=True):
             lam = W[p + "vmix"].to(F64)
             v = (1 - lam) * v + lam * v_first
     fn = sink_attention_fast if fast else sink_attention
-    o = fn(q, k, v, W[p + "rel"].to(F64), H, G, m["scale"], m["mask"]["size"], m["bias_max"])
+    chunk = (m.get("mask") or {}).get("size") or (1 << 30)
+    o = fn(q, k, v, W[p + "rel"].to(F64), H, G, m["scale"], chunk, m["bias_max"])
     return o @ W[p + "o"].to(F64).t(), mine
 
 
@@ -148,6 +150,7 @@ def hyper_sublayer(xs, W, p, norm_w, eps, fn):
 
 
 def forward(cfg, W, tokens, fast=True):
+    """A checkpoint without stream weights (one stream) takes the plain residual x + sublayer(norm(x))."""
     eps = cfg["norm"]["eps"]
     x = embed(W, tokens)
     S = int(cfg.get("streams", 1))
@@ -161,7 +164,7 @@ def forward(cfg, W, tokens, fast=True):
             y, mine = attention_mixer(lc["mixer"], W, p + "mix.", h, eps, v_first, fast)
             state["mine"] = mine
             return y
-        if S > 1:
+        if p + "hc1.in" in W:
             xs = hyper_sublayer(xs, W, p + "hc1.", W[p + "norm1"].to(F64), eps, mixer)
         else:
             xs = xs + mixer(rms(xs[0], W[p + "norm1"].to(F64), eps))[None]
@@ -171,7 +174,7 @@ def forward(cfg, W, tokens, fast=True):
         if mlp is not None:
             ff = (lambda h: dense_ff(mlp, W, p + "mlp.", h)) if mlp.get("kind", "dense") == "dense" else \
                 (lambda h: moe_ff(mlp, W, p + "mlp.", h))
-            if S > 1:
+            if p + "hc2.in" in W:
                 xs = hyper_sublayer(xs, W, p + "hc2.", W[p + "norm2"].to(F64), eps, ff)
             else:
                 xs = xs + ff(rms(xs[0], W[p + "norm2"].to(F64), eps))[None]
