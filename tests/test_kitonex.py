@@ -229,7 +229,7 @@ def test_router_choices(device):
     from llm_in_practise_amd.ops.moe import route_grouped
     z = torch.tensor([[3.0, -4.0, -4.0, 1.0, 1.2, -3.0, 2.0, 1.9, -9.0],      # groups of 3: sums 0.99, 1.50, 1.75
                       [0.1, 0.2, 0.3, 2.5, -5.0, -5.0, 0.0, 0.05, -0.1]]).to(device)
-    idx, w = route_grouped(z, None, 2, 3, 1, 1.0, score="sigmoid", group_rank="top2", normalize=True)
+    idx, w = (t.cpu() for t in route_grouped(z, None, 2, 3, 1, 1.0, score="sigmoid", group_rank="top2", normalize=True))
     assert idx.tolist() == [[6, 7], [2, 1]]
     s = torch.sigmoid(z.cpu().double())
     for t in range(2):
@@ -238,7 +238,7 @@ def test_router_choices(device):
         assert idx[t].tolist() == O.choose_experts(s[t], 2, 3, 1)
     idx, _ = route_grouped(z, None, 3, 3, 2, 1.0, score="sigmoid", group_rank="top2", normalize=True)
     assert idx.tolist() == [[6, 7, 4], [2, 1, 0]]
-    idx, w = route_grouped(z, None, 2, 3, 1, 1.0, score="sigmoid", group_rank="max", normalize=False)
+    idx, w = (t.cpu() for t in route_grouped(z, None, 2, 3, 1, 1.0, score="sigmoid", group_rank="max", normalize=False))
     assert idx.tolist()[0] == [0, 1] and abs(w[0, 0].item() - s[0, 0].item()) < 1e-6
 
 
@@ -620,4 +620,4 @@ def test_expert_paths_agree():
     sh, sg = torch.randn(T, W_, generator=g).cuda(), torch.randn(T, generator=g).cuda()
     a = moe_glu_experts(h, wgu, wd, idx, w, 0.0, sh, True, act="silu", shared_gate=sg)
     b = moe_glu_experts(h, wgu, wd, idx, w, 0.0, sh, False, act="silu", shared_gate=sg)
-    close(a, b.double(), 1e-5)
+    close(a, b.double().cpu(), 1e-5)
