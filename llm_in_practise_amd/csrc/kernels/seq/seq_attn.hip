@@ -135,6 +135,9 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
   const int blk = GQA ? x.block : 0;
   const int lo_t = blk > 0 ? ((HEADS ? pos_q : d.tok_pos[t0]) / blk) * blk : 0, lo_q = blk > 0 ? (pos_q / blk) * blk : 0;
   const float* brow = (GQA && x.bias != nullptr) ? x.bias + (size_t)g * x.nd : nullptr;
+  // a tile's queries sit at consecutive positions p0 + ql, so a 32-key tile meets only the 63 distances
+  // p0 - jb - 31 + i: lane i fetches that one bias and the 16 a lane needs come from its neighbours' registers
+  const int p0 = HEADS ? pos_q : d.tok_pos[t0];
   const float sl2 = scale * 1.4426950408889634f;   // scores in units of log2: v_exp_f32 is 2^x
   const int trow = 4 * (lane >> 5) + ((lane & 15) >> 2), tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   const int per = (pmax - lo_t + nsplit) / nsplit, j0 = lo_t + z * per, j1 = min(pmax + 1, j0 + per);
@@ -199,13 +202,16 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
     for (int ds = 0; ds < NDS; ++ds)
       if (ds < nds)
         sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kr + 16 * ds), qf[ds], sc, 0, 0, 0);
-    float mt = -INFINITY;
+    float mt = -INFINITY, bw = 0.f;
+    if (GQA && !HEADS && brow != nullptr)
+      bw = brow[min(max(p0 - jb - 31 + lane, 0), x.nd - 1)] * 1.4426950408889634f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int key = jb + (r & 3) + 8 * (r >> 2) + 4 * hi;
+      const int kk = (r & 3) + 8 * (r >> 2) + 4 * hi, key = jb + kk;
       const bool seen = key <= pos_q && key < j1 && (!GQA || key >= lo_q);
       float v = sc[r] * sl2;
-      if (GQA && brow != nullptr && seen) v += brow[min(pos_q - key, x.nd - 1)] * 1.4426950408889634f;
+      if (GQA && !HEADS && brow != nullptr) v += __shfl(bw, ql - kk + 31, 64);
+      if (GQA && HEADS && brow != nullptr && seen) v += brow[min(pos_q - key, x.nd - 1)] * 1.4426950408889634f;
       sc[r] = seen ? v : -INFINITY;
       mt = fmaxf(mt, sc[r]);
     }

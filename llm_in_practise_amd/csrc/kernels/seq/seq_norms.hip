@@ -348,6 +348,92 @@ __global__ __launch_bounds__(256) void k_hyper_mix_norm(float* __restrict__ X, c
   }
 }
 
+// The same with four columns per thread and 16-byte accesses; the mixed columns a thread has read stay in its
+// registers for the write after the reduction (widths up to 4 * 256 * HUC; wider rows re-read the rest).
+constexpr int HUC = 4;
+__device__ __forceinline__ f32x4 ld4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 ld4(const bf16* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+__device__ __forceinline__ void st4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16* p, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+}
+
+template <typename T, typename YT>
+__global__ __launch_bounds__(256) void k_hyper_mix_norm4(float* __restrict__ X, const YT* __restrict__ y, int ldy,
+                                                         const float* __restrict__ mix, const float* __restrict__ outw,
+                                                         const float* __restrict__ read, const float* __restrict__ w,
+                                                         T* __restrict__ h, int W, int S, float eps) {
+  __shared__ float sc[4];
+  __shared__ float sm[MAXS * MAXS + 2 * MAXS];
+  const size_t t = blockIdx.x;
+  float* smix = sm;
+  float* sout = sm + MAXS * MAXS;
+  float* srd = sout + MAXS;
+  if (threadIdx.x < S * S) smix[threadIdx.x] = y != nullptr ? mix[threadIdx.x] : 0.f;
+  if (threadIdx.x < S) {
+    sout[threadIdx.x] = y != nullptr ? outw[threadIdx.x] : 0.f;
+    srd[threadIdx.x] = read[threadIdx.x];
+  }
+  __syncthreads();
+  float* xr = X + t * S * W;
+  const int W4 = W >> 2;
+  // four columns: streams mixed and written back (with y), their read-weighted sum returned
+  auto columns = [&](int c4) -> f32x4 {
+    f32x4 old[MAXS], u = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s)
+      if (s < S) old[s] = ld4(xr + (size_t)s * W + 4 * c4);
+    if (y != nullptr) {
+      const f32x4 yv = ld4(y + t * ldy + 4 * c4);
+#pragma unroll
+      for (int k = 0; k < MAXS; ++k)
+        if (k < S) {
+          f32x4 v = yv * sout[k];
+#pragma unroll
+          for (int s = 0; s < MAXS; ++s)
+            if (s < S) v += old[s] * smix[s * S + k];
+          st4(xr + (size_t)k * W + 4 * c4, v);
+          u += v * srd[k];
+        }
+    } else {
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s)
+        if (s < S) u += old[s] * srd[s];
+    }
+    return u;
+  };
+  f32x4 keep[HUC];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < HUC; ++i) {
+    const int c4 = threadIdx.x + 256 * i;
+    if (c4 < W4) {
+      keep[i] = columns(c4);
+      ss += keep[i][0] * keep[i][0] + keep[i][1] * keep[i][1] + keep[i][2] * keep[i][2] + keep[i][3] * keep[i][3];
+    }
+  }
+  for (int c4 = threadIdx.x + 256 * HUC; c4 < W4; c4 += 256) {
+    const f32x4 u = columns(c4);
+    ss += u[0] * u[0] + u[1] * u[1] + u[2] * u[2] + u[3] * u[3];
+  }
+  const float rs = rsqrtf(block_sum256(ss, sc) / W + eps);
+#pragma unroll
+  for (int i = 0; i < HUC; ++i) {
+    const int c4 = threadIdx.x + 256 * i;
+    if (c4 < W4) st4(h + t * W + 4 * c4, keep[i] * ld4(w + 4 * c4) * rs);
+  }
+  for (int c4 = threadIdx.x + 256 * HUC; c4 < W4; c4 += 256) {      // the thread re-reads the columns it wrote itself
+    f32x4 u = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s)
+      if (s < S) u += ld4(xr + (size_t)s * W + 4 * c4) * srd[s];
+    st4(h + t * W + 4 * c4, u * ld4(w + 4 * c4) * rs);
+  }
+}
+
 // A step's [q | k | v] rows on their way into attention: q and k RMS-normed over their whole width, the normed k and
 // the values (blended with another cache's values of the same slot and position when vfirst is given:
 // (1 - lam) v + lam vfirst) written to the slot cache rows of each token's position.
@@ -491,8 +577,15 @@ void seq_embed_learned(int code, const long* tok, const int* pos, const void* ta
 void seq_hyper_mix_norm(int code, int y_f32, float* X, const void* y, int ldy, const float* mix, const float* outw,
                         const float* read, const float* w, void* h, int T_, int W, int S, float eps, hipStream_t st) {
   if (T_ == 0) return;
+  const bool vec = W % 4 == 0 && ldy % 4 == 0 && ((uintptr_t)y & 15) == 0;      // 16-byte rows (X, w, h are whole tensors)
   SEQ_DISPATCH_T(code, {
-    if (y_f32)
+    if (vec && y_f32)
+      hipLaunchKernelGGL((k_hyper_mix_norm4<T, float>), dim3(T_), dim3(256), 0, st, X, (const float*)y, ldy, mix, outw,
+                         read, w, (T*)h, W, S, eps);
+    else if (vec)
+      hipLaunchKernelGGL((k_hyper_mix_norm4<T, T>), dim3(T_), dim3(256), 0, st, X, (const T*)y, ldy, mix, outw, read, w,
+                         (T*)h, W, S, eps);
+    else if (y_f32)
       hipLaunchKernelGGL((k_hyper_mix_norm<T, float>), dim3(T_), dim3(256), 0, st, X, (const float*)y, ldy, mix, outw,
                          read, w, (T*)h, W, S, eps);
     else
