@@ -342,7 +342,15 @@ static bool sweep(int code, const void* q, int ldq, const void* kc, int ldk, con
   hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS, NW, GQA>), grid, dim3(64 * NW), 0, st, (const bf16*)q, ldq,  \
                      (const bf16*)kc, (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, ldk, ldv, max_len, \
                      nsplit, scale, d, x)
-    if (dk <= 128 && dv <= 128) {
+    bool small = false;                            // small heads: half the accumulators, more waves per SIMD
+    if constexpr (GQA) {
+      small = dk <= 64 && dv <= 64;
+      if (small) {
+        if (heads) SEQ_ATTN_LAUNCH(4, 2, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(4, 2, false, 4); else SEQ_ATTN_LAUNCH(4, 2, false, 1);
+      }
+    }
+    if (small) {
+    } else if (dk <= 128 && dv <= 128) {
       if (heads) SEQ_ATTN_LAUNCH(8, 4, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(8, 4, false, 4); else SEQ_ATTN_LAUNCH(8, 4, false, 1);
     } else {
       if (heads) SEQ_ATTN_LAUNCH(16, 8, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(16, 8, false, 4); else SEQ_ATTN_LAUNCH(16, 8, false, 1);

@@ -462,6 +462,17 @@ def test_bf16_matrix_core_sizes_long_context(device, heads, kv_heads, block):
     close(got, logits_of(cfg, W, toks), 0.06)
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_bf16_matrix_core_large_heads(device):
+    """Heads of 128 and beyond (the sweep's wider forms), a block edge inside a 32-query tile."""
+    cfg = config([attn(heads=4, kv_heads=1, dim=128, vdim=128, block=50, far=60, v_mix=False, mlp=dense()),
+                  attn(heads=2, kv_heads=1, dim=144, vdim=160, block=70, far=60, v_mix=False)], width=64, max_positions=160)
+    lm, W = build(cfg, device, 27, dtype=torch.bfloat16, tweak=_far_bias(2, 4.0))
+    toks = tokens(150, cfg["vocab"], 28)
+    got = replay(lm, 300, [([("a", toks[:140])], [])] + [([("a", [t])], []) for t in toks[140:]])["a"]
+    close(got, logits_of(cfg, W, toks), 0.06)
+
+
 def test_checkpoint_roundtrip_and_registry(tmp_path):
     from safetensors.torch import save_file
     from llm_in_practise_amd.models.registry import load_causal_lm
