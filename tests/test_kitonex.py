@@ -463,6 +463,21 @@ def test_bf16_matrix_core_sizes_long_context(device, heads, kv_heads, block):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_bf16_matrix_core_unequal_batch(device):
+    """Prompts of 1, 40, 97 and 130 tokens packed into one step (tiles of one sequence never cross into the next),
+    then decoded together, on sizes the matrix-core sweep takes."""
+    cfg = config([attn(heads=8, kv_heads=2, dim=32, vdim=32, block=48, far=50, mlp=dense()),
+                  attn(heads=8, kv_heads=2, dim=32, vdim=32, block=48, far=50, mlp=moe(experts=4, top=4))], width=64,
+                 max_positions=160)
+    lm, W = build(cfg, device, 29, dtype=torch.bfloat16, tweak=_far_bias(2, 4.0))
+    reqs = {i: tokens(n + 6, cfg["vocab"], 30 + n) for i, n in (("a", 1), ("b", 40), ("c", 97), ("d", 130))}
+    steps = [([(i, t[:-6]) for i, t in reqs.items()], [])] + [([(i, [t[j - 6]]) for i, t in reqs.items()], []) for j in range(6)]
+    got = replay(lm, 600, steps)
+    for i, t in reqs.items():
+        close(got[i], logits_of(cfg, W, t), 0.06)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_bf16_matrix_core_large_heads(device):
     """Heads of 128 and beyond (the sweep's wider forms), a block edge inside a 32-query tile."""
     cfg = config([attn(heads=4, kv_heads=1, dim=128, vdim=128, block=50, far=60, v_mix=False, mlp=dense()),
