@@ -211,7 +211,10 @@ def distance_bias_table(rel: torch.Tensor, far: float, distances: int) -> torch.
     import math
     B = rel.shape[0]
     half = B // 2
-    ids = [n if n < half else min(B - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (B - half))))
+    # (a distance that sits exactly on a bucket's lower edge belongs to that bucket: rounding in the logarithms must
+    # not push it one down, hence the 1e-9)
+    ids = [n if n < half else
+           min(B - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (B - half) + 1e-9)))
            for n in range(distances)]
     return rel.float()[torch.tensor(ids, dtype=torch.long, device=rel.device)].t().contiguous()
 

@@ -40,7 +40,8 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
     half = rows // 2
     if n < half:
         return n
-    return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half))))
+    x = math.log(n / half) / math.log(far / half) * (rows - half)
+    return min(rows - 1, half + int(math.floor(x + 1e-9)))          # an exact edge is not lost to rounding
 
 
 def sink_attention(q, k, v, rel, H, G, scale, chunk, far):

@@ -171,13 +171,15 @@ def test_attention_alone(device, kw):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("rows,far", [(10, 40), (2, 3), (32, 240), (16, 8.5), (64, 100)])
+@pytest.mark.parametrize("rows,far", [(10, 40), (2, 3), (32, 240), (16, 8.5), (64, 100), (10, 160), (32, 256)])
 def test_distance_bias_buckets(device, rows, far):
     from llm_in_practise_amd.ops.attention import distance_bias_table
     rel = torch.randn(rows, 3, generator=torch.Generator().manual_seed(rows)).to(device)
     tab = distance_bias_table(rel, far, 300).cpu()
     for n in range(300):
         assert torch.equal(tab[:, n], rel[O.distance_bucket(n, rows, far)].cpu()), n
+    if (rows, far) == (10, 160):                      # edges at 5 * 2^k: 10, 20, 40, 80 start buckets 6, 7, 8, 9
+        assert [O.distance_bucket(n, rows, far) for n in (9, 10, 19, 20, 39, 40, 79, 80, 159, 160)] == [5, 6, 6, 7, 7, 8, 8, 9, 9, 9]
     # the model keeps only the distances its block can show, or up to where the buckets end
     _check(device, [attn(block=0, far=far)], T=60, decode_from=50, wkw=dict(rows=rows))
 
