@@ -30,11 +30,17 @@ def _kitonex():
     return KitonexForCausalLM
 
 
+def _mamivik():
+    from .mamivik import MamivikForCausalLM
+    return MamivikForCausalLM
+
+
 REGISTRY = {
     "qwen3": _qwen, "qwen2": _qwen, "qwen3forcausallm": _qwen, "qwen2forcausallm": _qwen,
     "mobupel": _mobupel, "mobupelforcausallm": _mobupel,
     "dogudra": _dogudra, "dogudraforcausallm": _dogudra,
     "kitonex": _kitonex, "kitonexforcausallm": _kitonex,
+    "mamivik": _mamivik, "mamivikforcausallm": _mamivik,
 }
 
 

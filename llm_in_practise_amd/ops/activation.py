@@ -83,3 +83,22 @@ def silu_glu(z: torch.Tensor) -> torch.Tensor:
     if use_seq(z):
         return native_seq().ff_act(z.contiguous(), 2, 0.0)
     return ref.silu_glu(z)
+
+
+def gelu_glu(z: torch.Tensor) -> torch.Tensor:
+    """``z = [gate | up]``: ``gelu_tanh(gate) * up``."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(z):
+        return native_seq().ff_act(z.contiguous(), 3, 0.0)
+    return ref.gelu_glu(z)
+
+
+def sigmoid_gate(y: torch.Tensor, gate_pre: torch.Tensor) -> torch.Tensor:
+    """``y * sigmoid(gate_pre)`` element by element (``gate_pre`` may be a column slice of a wider matrix); the
+    sigmoid and the product are float."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(y):
+        return native_seq().sigmoid_gate(y, gate_pre)
+    return ref.sigmoid_gate(y, gate_pre)

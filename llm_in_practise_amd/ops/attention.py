@@ -177,30 +177,57 @@ def rotary_inv_freq(dims: int, base: float) -> torch.Tensor:
     return (float(base) ** (-2.0 * i / max(dims, 1))).float()
 
 
+def rotary_table(dims: int, base: float, scaling: dict | None = None) -> tuple[torch.Tensor, float]:
+    """Rotation frequencies ``[dims / 2]`` (float) and the magnitude that sine and cosine carry.  Without ``scaling``:
+    ``base^(-2i / dims)`` and 1.  With ``scaling = {factor, original, fast, slow}`` (long-context interpolation by
+    parts): a frequency that turns more than ``fast`` times over ``original`` positions stays, one that turns fewer
+    than ``slow`` times is divided by ``factor``, those between are blended linearly in the dimension index; the
+    magnitude is ``0.1 ln(factor) + 1``.  Evaluated in float64 on the host, rounded once."""
+    f = rotary_inv_freq(dims, base).double()
+    if not scaling:
+        return f.float(), 1.0
+    factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+    def dim_of(turns: float) -> float:
+        return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+    lo = max(math.floor(dim_of(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(dim_of(float(scaling["slow"]))), dims - 1)
+    ramp = ((torch.arange(dims // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return (f / factor * ramp + f * (1.0 - ramp)).float(), 0.1 * math.log(factor) + 1.0
+
+
 def latent_kv_store(u: torch.Tensor, norm_weight: torch.Tensor, inv_freq: torch.Tensor, cache: torch.Tensor,
-                    rot_dims: int, eps: float, sb) -> None:
+                    rot_dims: int, eps: float, sb, half: bool = False, mag: float = 1.0) -> None:
     """Writes a step's rows of a latent attention cache ``[slots, max_len, R + dr]``: ``u`` ``[T, R + dr]`` is the
     down-projection; its first ``R`` entries are RMS-normed (``norm_weight``), its last ``dr`` are the key part shared
-    by all heads, rotated pairwise (neighbours ``2i, 2i+1`` below ``rot_dims``) at each token's position."""
+    by all heads, rotated at each token's position: neighbours ``2i, 2i+1`` below ``rot_dims``, or with ``half``
+    entries ``i, i + rot_dims/2``; sine and cosine are multiplied by ``mag``."""
     from ._native import native_seq, use_seq
     if use_seq(u):
-        return native_seq().latent_kv_store(u, norm_weight, inv_freq, cache, rot_dims, eps, sb.desc)
-    return ref.latent_kv_store(u, norm_weight, inv_freq, cache, rot_dims, eps, sb)
+        return native_seq().latent_kv_store(u, norm_weight, inv_freq, cache, rot_dims, eps, sb.desc, half, mag)
+    return ref.latent_kv_store(u, norm_weight, inv_freq, cache, rot_dims, eps, sb, half, mag)
 
 
 def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, gate_pre: torch.Tensor | None,
                      inv_freq: torch.Tensor, heads: int, dim: int, rot_dims: int, scale: float, sb,
-                     nsplit: int = 1) -> torch.Tensor:
+                     nsplit: int = 1, half: bool = False, mag: float = 1.0, window: int = 0,
+                     sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Causal softmax attention of ``heads`` query heads over ONE shared row per key position, ``[c | kr]``:
     ``score_h = (q_abs_h . c + rot(q_rot_h) . kr) * scale``, result ``sum_j w_h(j) c(j)`` times
     ``sigmoid(gate_pre[t, h])``.  ``q_abs`` ``[H, T, R]`` holds the unrotated query parts already carried through the
     key up-projection; ``q`` ``[T, H*(dim + dr)]`` supplies the rotated parts (rotated here).  Returns ``[T, H, R]``;
-    the caller applies the value up-projection.  Scores and weights are float."""
+    the caller applies the value up-projection.  Scores and weights are float.  ``half`` / ``mag``: the rotation's
+    layout and magnitude as in :func:`latent_kv_store`.  ``window > 0``: a query sees only the keys less than ``window``
+    positions back (itself included); ``sinks`` float ``[H]``: ``exp(sinks[h])`` joins head ``h``'s denominators (a
+    key without a value).  With a window or sinks the gate must be applied by the caller."""
     from ._native import native_seq, use_seq
+    if (window > 0 or sinks is not None) and gate_pre is not None:
+        raise ValueError("latent_attention: a per-head gate is not combined with a window or sinks")
     if use_seq(q):
         return native_seq().latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, nsplit,
-                                             sb.desc, sb.tiles)
-    return ref.latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, sb)
+                                             sb.desc, sb.tiles, half, mag, window, sinks)
+    return ref.latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, sb, half, mag, window,
+                                sinks)
 
 
 def distance_bias_table(rel: torch.Tensor, far: float, distances: int) -> torch.Tensor:
@@ -233,17 +260,39 @@ def qk_norm_store(u: torch.Tensor, nq: int, nk: int, q_weight: torch.Tensor, k_w
     return ref.qk_norm_store(u, nq, nk, q_weight, k_weight, k_cache, v_cache, v_first, lam, eps, sb)
 
 
+def rope_kv_store(u: torch.Tensor, nq: int, nk: int, heads: int, kv_heads: int, inv_freq: torch.Tensor, rot_dims: int,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, sb, half: bool = True, mag: float = 1.0,
+                  values_are_keys: bool = False) -> torch.Tensor:
+    """The step's ``[q | k (| v)]`` rows ``u`` on their way into rotary attention: the first ``rot_dims`` entries of
+    every q and k head are rotated at the token's position (``half``: entries ``i, i + rot_dims/2`` form a pair, else
+    neighbours; ``mag`` multiplies sine and cosine); the rotated k goes to ``k_cache`` ``[slots, max_len, nk]`` at each
+    token's slot and position; ``v_cache`` gets ``u``'s v columns or, with ``values_are_keys``, the k columns as they
+    came (unrotated).  Angles and the rotation are float.  Returns the rotated q ``[T, nq]``."""
+    from ._native import native_seq, use_seq
+    if use_seq(u):
+        return native_seq().rope_kv_store(u, nq, nk, heads, kv_heads, inv_freq, rot_dims, k_cache, v_cache, sb.desc, half,
+                                          mag, values_are_keys)
+    return ref.rope_kv_store(u, nq, nk, heads, kv_heads, inv_freq, rot_dims, k_cache, v_cache, sb, half, mag,
+                             values_are_keys)
+
+
 def biased_attention(q, k_cache, v_cache, bias: torch.Tensor | None, heads: int, kv_heads: int, scale: float, sb,
-                     block: int = 0, sink: float | None = None, nsplit: int = 1):
+                     block: int = 0, sink: float | torch.Tensor | None = None, nsplit: int = 1, window: int = 0,
+                     out: torch.Tensor | None = None, out_scale: float = 1.0):
     """Causal grouped-query softmax attention over a slot-indexed cache with three optional parts:
     ``bias`` float ``[H, ND]`` adds ``bias[h, min(i - j, ND - 1)]`` to the scaled score of query ``i`` and key ``j``
     (``scale`` does not multiply it); ``block > 0`` lets a query see only keys of its own run of ``block`` positions
     (runs counted from the sequence's position 0); ``sink`` adds one key of that score and no value to every
     softmax (``0.0``: one is added to the denominator).  ``q`` ``[T, H*dk]`` for the step's packed tokens; the caches
     ``[slots, max_len, G*dk | G*dv]`` already hold the step's rows.  Returns ``[T, H*dv]``; scores and weights are
-    float.  ``nsplit`` cuts each query's keys into that many independent sweeps (decode)."""
+    float.  ``nsplit`` cuts each query's keys into that many independent sweeps (decode).  ``sink`` may be a float
+    tensor ``[H]``: one score per head.  ``window > 0``: a query sees only the keys less than ``window`` positions
+    back (itself included).  ``out`` (``[T, H*dv]``, a column slice of a wider matrix is fine) receives the result,
+    multiplied by ``out_scale``."""
     from ._native import native_seq, use_seq
     if use_seq(q):
+        per_head = sink if torch.is_tensor(sink) else None
         return native_seq().biased_attention(q, k_cache, v_cache, bias, heads, kv_heads, scale, block,
-                                             sink is not None, float(sink or 0.0), nsplit, sb.desc, sb.tiles)
-    return ref.biased_attention(q, k_cache, v_cache, bias, heads, kv_heads, scale, block, sink, sb)
+                                             sink is not None, 0.0 if per_head is not None else float(sink or 0.0),
+                                             nsplit, sb.desc, sb.tiles, window, per_head, out, out_scale)
+    return ref.biased_attention(q, k_cache, v_cache, bias, heads, kv_heads, scale, block, sink, sb, window, out, out_scale)

@@ -144,17 +144,19 @@ def dual_norm_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor, eps: float,
-                   den: torch.Tensor | None = None, floor: torch.Tensor | None = None) -> torch.Tensor:
+                   den: torch.Tensor | None = None, floor: torch.Tensor | None = None,
+                   out: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
     """Read-out of a recurrent mixer: ``o`` float ``[T, H, dv]`` is RMS-normed per head, scaled by ``weight``
     (``[dv]`` shared by the heads or ``[H * dv]``) and multiplied by ``sigmoid(gate_pre)``; returns ``[T, H * dv]``
     in ``gate_pre``'s dtype.  With ``den`` / ``floor`` (float ``[T, H]``) ``o`` is first divided by
-    ``max(|den|, floor) + 1e-6`` (the mLSTM's normaliser)."""
+    ``max(|den|, floor) + 1e-6`` (the mLSTM's normaliser).  ``out`` (``[T, H * dv]``, a column slice of a wider matrix
+    is fine) receives the result, multiplied by ``scale``."""
     from ._native import native_seq, use_seq
     if use_seq(o):
-        return native_seq().head_norm_gate(o, weight, gate_pre, eps, den, floor)
+        return native_seq().head_norm_gate(o, weight, gate_pre, eps, den, floor, out, scale)
     if den is not None:
         o = o / (torch.maximum(den.abs(), floor) + 1e-6)[..., None]
-    return ref.head_norm_gate(o, weight, gate_pre, eps)
+    return ref.head_norm_gate(o, weight, gate_pre, eps, out, scale)
 
 
 def scaled_postnorm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, alpha: float, eps: float,

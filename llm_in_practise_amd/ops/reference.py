@@ -183,10 +183,14 @@ def polynorm(z, coef, eps: float):
     return out.to(z.dtype)
 
 
-def head_norm_gate(o, w, gate, eps: float):
+def head_norm_gate(o, w, gate, eps: float, out=None, scale: float = 1.0):
     T, H, dv = o.shape
     y = _unit_rms(o, eps) * (w.view(H, dv) if w.numel() != dv else w)
-    return (y.reshape(T, H * dv) * torch.sigmoid(gate.float())).to(gate.dtype)
+    y = y.reshape(T, H * dv) * torch.sigmoid(gate.float()) * scale
+    if out is None:
+        return y.to(gate.dtype)
+    out.copy_(y)
+    return out
 
 
 def decay_gate(pre, bias, a_log, dk: int):
@@ -364,17 +368,43 @@ def rotate_pairs(v, pos, inv_freq, dims: int):
     return out
 
 
-def latent_kv_store(u, w, inv_freq, cache, dims: int, eps: float, sb):
+def rotate_halves(v, pos, inv_freq, dims: int, mag: float = 1.0):
+    """v [T, ..., d] float: entries (i, i + dims/2), i < dims/2, turn by pos * inv_freq[i]; sine and cosine carry
+    ``mag``."""
+    if dims == 0:
+        return v
+    half = dims // 2
+    ang = pos.float().reshape(-1, *([1] * (v.dim() - 1))) * inv_freq[:half].float()
+    c, s = torch.cos(ang) * mag, torch.sin(ang) * mag
+    a, b = v[..., :half], v[..., half:dims]
+    out = v.clone()
+    out[..., :half] = a * c - b * s
+    out[..., half:dims] = b * c + a * s
+    return out
+
+
+def rotate(v, pos, inv_freq, dims: int, half: bool = False, mag: float = 1.0):
+    if half:
+        return rotate_halves(v, pos, inv_freq, dims, mag)
+    out = rotate_pairs(v, pos, inv_freq, dims)
+    if mag != 1.0 and dims:
+        out = out.clone()
+        out[..., :dims] = out[..., :dims] * mag
+    return out
+
+
+def latent_kv_store(u, w, inv_freq, cache, dims: int, eps: float, sb, half: bool = False, mag: float = 1.0):
     R = w.numel()
     c = _unit_rms(u[:, :R].float(), eps) * w
-    kr = rotate_pairs(u[:, R:].float(), sb.desc[4], inv_freq, dims)
+    kr = rotate(u[:, R:].float(), sb.desc[4], inv_freq, dims, half, mag)
     cache.view(-1, cache.shape[2]).index_copy_(0, sb.cache_idx, torch.cat([c, kr], 1).to(cache.dtype))
 
 
-def latent_attention(qa, q, cache, gate, inv_freq, H: int, dn: int, dims: int, scale: float, sb):
+def latent_attention(qa, q, cache, gate, inv_freq, H: int, dn: int, dims: int, scale: float, sb, half: bool = False,
+                     mag: float = 1.0, window: int = 0, sinks=None):
     T, R = q.shape[0], qa.shape[2]
     dr = q.shape[1] // H - dn
-    qr = rotate_pairs(q.float().view(T, H, dn + dr)[..., dn:], sb.desc[4], inv_freq, dims)
+    qr = rotate(q.float().view(T, H, dn + dr)[..., dn:], sb.desc[4], inv_freq, dims, half, mag)
     Q = torch.cat([qa.transpose(0, 1).float(), qr], -1).to(q.dtype).float()       # [T, H, R + dr]
     out = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
     off, slots, pos0 = sb.host()
@@ -383,12 +413,29 @@ def latent_attention(qa, q, cache, gate, inv_freq, H: int, dn: int, dims: int, s
         L = pos0[b] + e - a
         rows = cache[slot, :L].float()
         sc = torch.einsum("thd,ld->htl", Q[a:e], rows) * scale
-        vis = torch.arange(L, device=q.device)[None, :] <= (pos0[b] + torch.arange(e - a, device=q.device))[:, None]
-        w = torch.softmax(sc.masked_fill(~vis[None], float("-inf")), -1)
+        dist = (pos0[b] + torch.arange(e - a, device=q.device))[:, None] - torch.arange(L, device=q.device)[None, :]
+        vis = dist >= 0
+        if window > 0:
+            vis &= dist < window
+        w = _softmax_with_sink(sc.masked_fill(~vis[None], float("-inf")), sinks)
         out[a:e] = torch.einsum("htl,lr->thr", w, rows[:, :R])
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[..., None]
     return out.to(q.dtype)
+
+
+def _softmax_with_sink(sc, sinks):
+    """Softmax over the last axis of ``sc`` ``[H, T, L]``; ``sinks`` ``[H]`` (or one number) adds ``exp(sink)`` to
+    every denominator of its head."""
+    m = sc.max(-1, keepdim=True).values
+    if sinks is not None:
+        sk = sinks.float().reshape(-1, 1, 1) if torch.is_tensor(sinks) else torch.full((1, 1, 1), float(sinks), device=sc.device)
+        m = torch.maximum(m, sk)
+    w = torch.exp(sc - m)
+    den = w.sum(-1, keepdim=True)
+    if sinks is not None:
+        den = den + torch.exp(sk - m)
+    return w / den
 
 
 def route_grouped(z, corr, top: int, groups: int, keep: int, scale: float):
@@ -431,11 +478,12 @@ def qk_norm_store(u, nq: int, nk: int, qw, kw, kc, vc, v_first, lam, eps: float,
     return q
 
 
-def biased_attention(q, kc, vc, bias, H: int, G: int, scale: float, block: int, sink, sb):
+def biased_attention(q, kc, vc, bias, H: int, G: int, scale: float, block: int, sink, sb, window: int = 0, out=None,
+                     out_scale: float = 1.0):
     T = q.shape[0]
     dk, dv = q.shape[1] // H, vc.shape[2] // G
     rep = H // G
-    out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+    res = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
     off, slots, pos0 = sb.host()
     for b, slot in enumerate(slots):
         a, e = off[b], off[b + 1]
@@ -449,18 +497,18 @@ def biased_attention(q, kc, vc, bias, H: int, G: int, scale: float, block: int, 
         vis = dist >= 0
         if block > 0:
             vis &= (qp[:, None] // block) == (kp[None, :] // block)
+        if window > 0:
+            vis &= dist < window
         if bias is not None:
             sc = sc + bias[:, dist.clamp(0, bias.shape[1] - 1)]
-        sc = sc.masked_fill(~vis[None], float("-inf"))
-        m = sc.max(-1, keepdim=True).values
-        if sink is not None:
-            m = m.clamp(min=float(sink))
-        w = torch.exp(sc - m)
-        den = w.sum(-1, keepdim=True)
-        if sink is not None:
-            den = den + torch.exp(float(sink) - m)
-        out[a:e] = torch.einsum("htl,lhd->thd", w / den, vv).reshape(e - a, H * dv)
-    return out.to(q.dtype)
+        w = _softmax_with_sink(sc.masked_fill(~vis[None], float("-inf")), sink)
+        res[a:e] = torch.einsum("htl,lhd->thd", w, vv).reshape(e - a, H * dv)
+    if out_scale != 1.0:
+        res = res * out_scale
+    if out is None:
+        return res.to(q.dtype)
+    out.copy_(res)
+    return out
 
 
 def route_scored(z, corr, top: int, groups: int, keep: int, scale: float, sigmoid: bool, top2: bool, normalize: bool):
@@ -483,3 +531,56 @@ def route_scored(z, corr, top: int, groups: int, keep: int, scale: float, sigmoi
 def silu_glu(z):
     F_ = z.shape[-1] // 2
     return (F.silu(z[..., :F_].float()) * z[..., F_:].float()).to(z.dtype)
+
+
+# ---- sliding-window attention whose values are its keys, generalised delta rule, GELU GLU, element-wise output gate
+def rope_kv_store(u, nq: int, nk: int, H: int, G: int, inv_freq, dims: int, kc, vc, sb, half: bool, mag: float,
+                  values_are_keys: bool):
+    T = u.shape[0]
+    dk = nq // H
+    pos = sb.desc[4]
+    q = rotate(u[:, :nq].float().view(T, H, dk), pos, inv_freq, dims, half, mag).reshape(T, nq).to(u.dtype)
+    k = rotate(u[:, nq:nq + nk].float().view(T, G, dk), pos, inv_freq, dims, half, mag).reshape(T, nk)
+    v = u[:, nq:nq + nk] if values_are_keys else u[:, nq + nk:]
+    kc.view(-1, nk).index_copy_(0, sb.cache_idx, k.to(kc.dtype))
+    vc.view(-1, vc.shape[2]).index_copy_(0, sb.cache_idx, v.to(vc.dtype))
+    return q
+
+
+def delta_rule_gates(k, w_low, w_up, w_bias, a_pre, a_bias, H: int, decay_scale: float):
+    T = k.shape[0]
+    dk = k.shape[1] // H
+    w_pre = w_low.float() if w_up is None else torch.tanh(w_low.float()) @ w_up.float().t()
+    w = torch.exp(-decay_scale * torch.sigmoid(w_pre + (w_bias if w_bias is not None else 0.0)))
+    a = torch.sigmoid(a_pre.float() + (a_bias if a_bias is not None else 0.0))
+    kf = k.float().view(T, H, dk)
+    u = (kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + 1e-6)).reshape(T, H * dk)
+    return w.contiguous(), u.contiguous(), (a * u).contiguous()
+
+
+def general_delta_scan(r, k, v, w, u, au, S, H: int, sb):
+    T = r.shape[0]
+    dk, dv = r.shape[1] // H, v.shape[1] // H
+    rf, kf, vf = r.float().view(T, H, dk), k.float().view(T, H, dk), v.float().view(T, H, dv)
+    wf, uf, af = w.view(T, H, dk), u.view(T, H, dk), au.view(T, H, dk)
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=r.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        if not sb.is_live(b):
+            continue
+        s = torch.zeros_like(S[slot]) if pos0[b] == 0 else S[slot].clone()   # [H, dv, dk]
+        for t in range(off[b], off[b + 1]):
+            d = (s * uf[t][:, None, :]).sum(-1)                              # [H, dv]: u^T S of the old state
+            s = s * wf[t][:, None, :] - d[:, :, None] * af[t][:, None, :] + vf[t][:, :, None] * kf[t][:, None, :]
+            out[t] = (s * rf[t][:, None, :]).sum(-1)
+        S[slot] = s
+    return out
+
+
+def gelu_glu(z):
+    F_ = z.shape[-1] // 2
+    return (F.gelu(z[..., :F_].float(), approximate="tanh") * z[..., F_:].float()).to(z.dtype)
+
+
+def sigmoid_gate(y, gate):
+    return (y.float() * torch.sigmoid(gate.float())).to(y.dtype)
