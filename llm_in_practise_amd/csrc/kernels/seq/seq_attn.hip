@@ -12,8 +12,11 @@
 // The same sweeps serve plain grouped-query attention (GQA = true): a query head meets only the values of its own kv
 // head, and three optional parts change which keys count and how: a float bias per (head, distance) added to the
 // scaled score, a block mask (a query sees only the keys of its own run of `block` positions, counted from the
-// sequence's position 0), and a sink (one more key of a fixed score without a value in every softmax).  With one key
-// split the matrix-core sweep normalises and writes the activation type itself; otherwise k_gqa_merge does.
+// sequence's position 0), a sliding window (a query sees only the keys less than `window` positions back, itself
+// included), and a sink (one more key of a fixed score, or of a learned score per head, without a value in every
+// softmax).  With one key split the matrix-core sweep normalises and writes the activation type itself; otherwise
+// k_gqa_merge does.  The output may be a column slice of a wider matrix (row stride ldo) and is multiplied by
+// out_scale.
 #include "seq_common.h"
 
 using namespace lipa;
@@ -23,9 +26,13 @@ struct GqaExtra {
   const float* bias;   // [H, nd] or null: bias[h][min(i - j, nd - 1)], in natural-log units
   int nd;
   int block;           // 0: every earlier key; > 0: keys of the query's own block
-  int sink;            // 1: a key of score sink_logit and no value
+  int sink;            // 1: a key of score sink_logit (or sinks[h]) and no value
   float sink_logit;
   void* out;           // [T, H * dv] in the activation type, written when nsplit == 1 (matrix-core sweep)
+  int window;          // 0: every earlier key; > 0: keys j with i - j < window
+  const float* sinks;  // [H] or null: a sink score per head, in place of sink_logit
+  int ldo;             // row stride of out
+  float out_scale;
 };
 
 constexpr int MAXC = 16;   // value columns per lane: G * dv <= 64 * MAXC
@@ -42,7 +49,8 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
   const int kh = g / (H / G), GV = GQA ? dv : G * dv;
   for (int i = lane; i < dk; i += 64) sq[i] = (float)q[(size_t)t * ldq + g * dk + i];
   __syncthreads();
-  const int lo = (GQA && x.block > 0) ? (p / x.block) * x.block : 0;
+  int lo = (GQA && x.block > 0) ? (p / x.block) * x.block : 0;
+  if (GQA && x.window > 0) lo = max(lo, p - x.window + 1);
   const int nkeys = p + 1 - lo, per = (nkeys + nsplit - 1) / nsplit;
   const int j0 = lo + z * per, j1 = min(p + 1, j0 + per);
   const T* kbase = kc + ((size_t)slot * max_len) * ldk + kh * dk;
@@ -132,8 +140,12 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
   const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, LDK = dk + 8, kh = HEADS ? blockIdx.y : g / rep;
   const int c = GQA ? kh : blockIdx.z % G, GV = GQA ? dv : G * dv;
   // block mask: the tile's sweep starts at the block of its first query; every query keeps its own block's keys
-  const int blk = GQA ? x.block : 0;
-  const int lo_t = blk > 0 ? ((HEADS ? pos_q : d.tok_pos[t0]) / blk) * blk : 0, lo_q = blk > 0 ? (pos_q / blk) * blk : 0;
+  const int blk = GQA ? x.block : 0, win = GQA ? x.window : 0;
+  int lo_t = blk > 0 ? ((HEADS ? pos_q : d.tok_pos[t0]) / blk) * blk : 0, lo_q = blk > 0 ? (pos_q / blk) * blk : 0;
+  if (win > 0) {                                   // sliding window: nothing before the first query's oldest key
+    lo_t = max(lo_t, (HEADS ? pos_q : d.tok_pos[t0]) - win + 1);
+    lo_q = max(lo_q, pos_q - win + 1);
+  }
   const float* brow = (GQA && x.bias != nullptr) ? x.bias + (size_t)g * x.nd : nullptr;
   // a tile's queries sit at consecutive positions p0 + ql, so a 32-key tile meets only the 63 distances
   // p0 - jb - 31 + i: lane i fetches that one bias and the 16 a lane needs come from its neighbours' registers
@@ -251,10 +263,11 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
   }
   if (!valid_q) return;
   if (GQA && nsplit == 1) {                      // the whole softmax is here: add the sink, normalise, write
-    const float sk = x.sink_logit * 1.4426950408889634f, mf = x.sink ? fmaxf(m, sk) : m;
+    const float sk = (x.sinks != nullptr ? x.sinks[g] : x.sink_logit) * 1.4426950408889634f, mf = x.sink ? fmaxf(m, sk) : m;
     const float e = mf == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mf);
-    const float den = l * e + (x.sink ? __builtin_amdgcn_exp2f(sk - mf) : 0.f), inv = den > 0.f ? e / den : 0.f;
-    bf16* orow = (bf16*)x.out + (size_t)tq * (H * dv) + g * dv;
+    const float den = l * e + (x.sink ? __builtin_amdgcn_exp2f(sk - mf) : 0.f);
+    const float inv = den > 0.f ? e / den * x.out_scale : 0.f;
+    bf16* orow = (bf16*)x.out + (size_t)tq * x.ldo + g * dv;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
       if (dt < ndt)
@@ -375,40 +388,46 @@ void seq_attn_sweep(int code, const void* q, int ldq, const void* kc, int ldk, c
                     float* pl, float* pu, int H, int G, int dk, int dv, int max_len, int nsplit, float scale,
                     const int* tile_seq, const int* tile_t0, int ntiles, SeqDesc d, hipStream_t st) {
   sweep<false>(code, q, ldq, kc, ldk, vc, ldv, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale, tile_seq, tile_t0,
-               ntiles, d, GqaExtra{nullptr, 0, 0, 0, 0.f, nullptr}, st);
+               ntiles, d, GqaExtra{nullptr, 0, 0, 0, 0.f, nullptr, 0, nullptr, 0, 1.f}, st);
 }
 
 // Merge of a GQA sweep's key splits: one wave per (token, head); the sink joins the denominator here.
 template <typename T>
 __global__ __launch_bounds__(64) void k_gqa_merge(const float* __restrict__ pm, const float* __restrict__ pl,
                                                   const float* __restrict__ pu, T* __restrict__ out, int H, int dv,
-                                                  int nsplit, int sink, float sink_logit) {
+                                                  int nsplit, int sink, float sink_logit,
+                                                  const float* __restrict__ sinks, int ldo, float out_scale) {
   const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
   const size_t b = ((size_t)t * H + g) * nsplit;
+  if (sinks != nullptr) sink_logit = sinks[g];
   float mx = sink ? sink_logit : -INFINITY;
   for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pm[b + z]);
   float l = sink ? expf(sink_logit - mx) : 0.f;
   for (int z = 0; z < nsplit; ++z) l += pm[b + z] == -INFINITY ? 0.f : expf(pm[b + z] - mx) * pl[b + z];
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float inv = l > 0.f ? out_scale / l : 0.f;
   for (int col = lane; col < dv; col += 64) {
     float u = 0.f;
     for (int z = 0; z < nsplit; ++z)
       if (pm[b + z] != -INFINITY) u += expf(pm[b + z] - mx) * pu[(b + z) * dv + col];
-    out[(size_t)t * (H * dv) + g * dv + col] = (T)(u * inv);
+    out[(size_t)t * ldo + g * dv + col] = (T)(u * inv);
   }
 }
 
-// Grouped-query attention over a slot-indexed cache with an optional distance bias, block mask and sink.
-void seq_gqa_attention(int code, const void* q, int ldq, const void* kc, const void* vc, float* pm, float* pl, float* pu,
-                       const float* bias, int nd, int block, int sink, float sink_logit, void* out, int H, int G, int dk,
-                       int dv, int max_len, int nsplit, float scale, const int* tile_seq, const int* tile_t0, int ntiles,
-                       SeqDesc d, hipStream_t st) {
+// Grouped-query attention over a slot-indexed cache with an optional distance bias, block mask, sliding window and
+// sink.  Key rows are ldk and value rows ldv elements apart (values may be columns of the key rows: a latent cache
+// with G = 1); the output rows are ldo elements apart.
+void seq_gqa_attention(int code, const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, float* pm,
+                       float* pl, float* pu, const float* bias, int nd, int block, int window, int sink, float sink_logit,
+                       const float* sinks, void* out, int ldo, float out_scale, int H, int G, int dk, int dv, int max_len,
+                       int nsplit, float scale, const int* tile_seq, const int* tile_t0, int ntiles, SeqDesc d,
+                       hipStream_t st) {
   if (d.Ttot == 0) return;
-  const bool direct = sweep<true>(code, q, ldq, kc, G * dk, vc, G * dv, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale,
-                                  tile_seq, tile_t0, ntiles, d, GqaExtra{bias, nd, block, sink, sink_logit, out}, st);
+  const bool direct = sweep<true>(code, q, ldq, kc, ldk, vc, ldv, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale,
+                                  tile_seq, tile_t0, ntiles, d,
+                                  GqaExtra{bias, nd, block, sink, sink_logit, out, window, sinks, ldo, out_scale}, st);
   if (direct) return;
   SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_gqa_merge<T>, dim3(d.Ttot, H), dim3(64), 0, st, pm, pl, pu, (T*)out, H, dv,
-                                          nsplit, sink, sink_logit));
+                                          nsplit, sink, sink_logit, sinks, ldo, out_scale));
   LIPA_CHECK_LAUNCH();
 }
 

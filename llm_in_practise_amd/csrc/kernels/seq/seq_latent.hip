@@ -10,23 +10,12 @@
 
 using namespace lipa;
 
-// neighbours (2i, 2i+1) of the first `dims` entries turn by pos * inv_freq[i]; the rest pass unchanged
-template <typename T>
-__device__ __forceinline__ float rotated_at(const T* __restrict__ v, int c, int n, int dims, float pos,
-                                            const float* __restrict__ inv_freq) {
-  const float a = (float)v[c];
-  if (c >= dims) return a;
-  const float b = (float)v[c ^ 1];
-  float sn, cs;
-  sincosf(pos * inv_freq[c >> 1], &sn, &cs);
-  return (c & 1) ? a * cs + b * sn : a * cs - b * sn;
-}
-
 // one block per token: row[0:R] = rms(u[0:R]) * w, row[R:R+dr] = rotate(u[R:R+dr]) at the token's position
 template <typename T>
 __global__ __launch_bounds__(256) void k_latent_kv_store(const T* __restrict__ u, int ldu, const float* __restrict__ w,
                                                          const float* __restrict__ inv_freq, T* __restrict__ cache,
-                                                         int R, int dr, int dims, int max_len, float eps, SeqDesc d) {
+                                                         int R, int dr, int dims, int max_len, float eps, int half,
+                                                         float mag, SeqDesc d) {
   __shared__ float sc[4];
   const int t = blockIdx.x, s = d.tok_seq[t], p = d.tok_pos[t], slot = d.slots[s];
   const T* src = u + (size_t)t * ldu;
@@ -38,7 +27,7 @@ __global__ __launch_bounds__(256) void k_latent_kv_store(const T* __restrict__ u
   }
   const float rs = rsqrtf(block_sum256(ss, sc) / R + eps);
   for (int c = threadIdx.x; c < R; c += 256) row[c] = (T)((float)src[c] * rs * w[c]);
-  for (int c = threadIdx.x; c < dr; c += 256) row[R + c] = (T)rotated_at(src + R, c, dr, dims, (float)p, inv_freq);
+  for (int c = threadIdx.x; c < dr; c += 256) row[R + c] = (T)rotated_at(src + R, c, dims, (float)p, inv_freq, half, mag);
 }
 
 // one block per (token, head): Q[t, h, 0:R] = qa[h, t, 0:R] (the absorbed unrotated part),
@@ -47,14 +36,15 @@ template <typename T>
 __global__ __launch_bounds__(128) void k_latent_q_assemble(const T* __restrict__ qa, size_t qa_sh, size_t qa_st,
                                                            const T* __restrict__ q, int ldq, int dn,
                                                            const float* __restrict__ inv_freq, T* __restrict__ out,
-                                                           int H, int R, int dr, int dims, SeqDesc d) {
+                                                           int H, int R, int dr, int dims, int half, float mag,
+                                                           SeqDesc d) {
   const int t = blockIdx.x, h = blockIdx.y;
   const float p = (float)d.tok_pos[t];
   T* dst = out + ((size_t)t * H + h) * (R + dr);
   const T* a = qa + h * qa_sh + t * qa_st;
   for (int c = threadIdx.x; c < R; c += 128) dst[c] = a[c];
   const T* r = q + (size_t)t * ldq + (size_t)h * (dn + dr) + dn;
-  for (int c = threadIdx.x; c < dr; c += 128) dst[R + c] = (T)rotated_at(r, c, dr, dims, p, inv_freq);
+  for (int c = threadIdx.x; c < dr; c += 128) dst[R + c] = (T)rotated_at(r, c, dims, p, inv_freq, half, mag);
 }
 
 // one block per (token, head): merge the key splits, normalise, multiply by sigmoid(gate[t, h]).  The splits' weights
@@ -95,18 +85,19 @@ __global__ __launch_bounds__(128) void k_latent_merge(const float* __restrict__ 
 }
 
 void seq_latent_kv_store(int code, const void* u, int ldu, const float* w, const float* inv_freq, void* cache, int R,
-                         int dr, int dims, int max_len, float eps, SeqDesc d, hipStream_t st) {
+                         int dr, int dims, int max_len, float eps, int half, float mag, SeqDesc d, hipStream_t st) {
   if (d.Ttot == 0) return;
   SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_latent_kv_store<T>, dim3(d.Ttot), dim3(256), 0, st, (const T*)u, ldu, w,
-                                          inv_freq, (T*)cache, R, dr, dims, max_len, eps, d));
+                                          inv_freq, (T*)cache, R, dr, dims, max_len, eps, half, mag, d));
   LIPA_CHECK_LAUNCH();
 }
 
 void seq_latent_q_assemble(int code, const void* qa, size_t qa_sh, size_t qa_st, const void* q, int ldq, int dn,
-                           const float* inv_freq, void* out, int H, int R, int dr, int dims, SeqDesc d, hipStream_t st) {
+                           const float* inv_freq, void* out, int H, int R, int dr, int dims, int half, float mag,
+                           SeqDesc d, hipStream_t st) {
   if (d.Ttot == 0) return;
   SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_latent_q_assemble<T>, dim3(d.Ttot, H), dim3(128), 0, st, (const T*)qa, qa_sh,
-                                          qa_st, (const T*)q, ldq, dn, inv_freq, (T*)out, H, R, dr, dims, d));
+                                          qa_st, (const T*)q, ldq, dn, inv_freq, (T*)out, H, R, dr, dims, half, mag, d));
   LIPA_CHECK_LAUNCH();
 }
 

@@ -232,8 +232,9 @@ __device__ __forceinline__ float clipped_glu(float g, float u, float limit) {
   return g * sigmoidf_(1.702f * g) * (u + 1.f);
 }
 
-// mode 1: the clipped GLU; mode 2: silu(g) * u
+// mode 1: the clipped GLU; mode 2: silu(g) * u; mode 3: gelu_tanh(g) * u
 __device__ __forceinline__ float glu(float g, float u, float limit, int mode) {
+  if (mode == 3) return gelu_tanhf_(g) * u;
   return mode == 2 ? g * sigmoidf_(g) * u : clipped_glu(g, u, limit);
 }
 
@@ -326,8 +327,8 @@ __global__ __launch_bounds__(256) void k_moe_combine(const T* __restrict__ ys, c
   }
 }
 
-// feed-forward activations on a GEMM output: mode 0 tanh-form GELU of z [T, F]; mode 1 clipped GLU, mode 2 SiLU GLU of
-// the [gate | up] halves of z [T, 2F]
+// feed-forward activations on a GEMM output: mode 0 tanh-form GELU of z [T, F]; mode 1 clipped GLU, mode 2 SiLU GLU,
+// mode 3 tanh-form GELU GLU of the [gate | up] halves of z [T, 2F]
 template <typename T>
 __global__ __launch_bounds__(256) void k_ff_act(const T* __restrict__ z, T* __restrict__ out, size_t n, int F, int mode,
                                                 float limit) {
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(256) void k_ff_act(const T* __restrict__ z, T* __re
   if (i >= n) return;
   if (mode == 0) {
     const float v = (float)z[i];
-    out[i] = (T)(0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v))));
+    out[i] = (T)gelu_tanhf_(v);
   } else {
     const size_t t = i / F, c = i % F;
     out[i] = (T)glu((float)z[t * 2 * F + c], (float)z[t * 2 * F + F + c], limit, mode);

@@ -107,7 +107,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void k_head_norm_gate(const float* __restrict__ o, const float* __restrict__ w,
                                                         int per_head, const T* __restrict__ gate, int ldg,
                                                         const float* __restrict__ den, const float* __restrict__ efl,
-                                                        T* __restrict__ out, int nrows, int H, int dv, float eps) {
+                                                        T* __restrict__ out, int ldo, float scale, int nrows, int H,
+                                                        int dv, float eps) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= nrows) return;
   const int t = row / H, hd = row % H;
@@ -120,8 +121,8 @@ __global__ __launch_bounds__(256) void k_head_norm_gate(const float* __restrict_
   }
   const float rs = rsqrtf(wave_sum(s) / dv + eps) * dinv;
   for (int c = lane; c < dv; c += 64) {
-    const float g = sigmoidf_((float)gate[(size_t)t * ldg + hd * dv + c]);
-    out[(size_t)row * dv + c] = (T)(src[c] * rs * w[(per_head ? hd * dv : 0) + c] * g);
+    const float g = sigmoidf_((float)gate[(size_t)t * ldg + hd * dv + c]) * scale;
+    out[(size_t)t * ldo + hd * dv + c] = (T)(src[c] * rs * w[(per_head ? hd * dv : 0) + c] * g);
   }
 }
 
@@ -465,6 +466,131 @@ __global__ __launch_bounds__(256) void k_qk_norm_store(const T* __restrict__ u, 
   }
 }
 
+// A step's [q | k (| v)] rows on their way into rotary attention: the first `dims` entries of every q and k head are
+// rotated at the token's position; the rotated k goes to the key cache; the value cache gets the v columns or, with
+// vkeys, the k columns as they came (a design whose values are its unrotated keys).  One block per token.
+template <typename T>
+__global__ __launch_bounds__(256) void k_rope_kv_store(const T* __restrict__ u, int ldu, const float* __restrict__ inv_freq,
+                                                       T* __restrict__ qout, T* __restrict__ kc, T* __restrict__ vc,
+                                                       int nq, int nk, int nv, int dk, int dims, int half, float mag,
+                                                       int vkeys, int max_len, SeqDesc d) {
+  const size_t t = blockIdx.x;
+  const T* r = u + t * ldu;
+  const int pos = d.tok_pos[t], slot = d.slots[d.tok_seq[t]];
+  const float p = (float)pos;
+  for (int c = threadIdx.x; c < nq; c += 256) {
+    const int cl = c % dk;
+    qout[t * nq + c] = (T)rotated_at(r + (c - cl), cl, dims, p, inv_freq, half, mag);
+  }
+  if (pos < 0 || pos >= max_len) return;             // a row nobody reads may carry any position
+  const size_t row = (size_t)slot * max_len + pos;
+  for (int c = threadIdx.x; c < nk; c += 256) {
+    const int cl = c % dk;
+    kc[row * nk + c] = (T)rotated_at(r + nq + (c - cl), cl, dims, p, inv_freq, half, mag);
+    if (vkeys) vc[row * nk + c] = r[nq + c];
+  }
+  if (!vkeys)
+    for (int c = threadIdx.x; c < nv; c += 256) vc[row * nv + c] = r[nq + nk + c];
+}
+
+// out = y * sigmoid(gate), element by element; gate rows are ldg apart
+template <typename T>
+__global__ __launch_bounds__(256) void k_sigmoid_gate(const T* __restrict__ y, const T* __restrict__ gate, int ldg,
+                                                      T* __restrict__ out, size_t n, int C) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const size_t t = i / C, c = i % C;
+  out[i] = (T)((float)y[i] * sigmoidf_((float)gate[t * ldg + c]));
+}
+
+// What the generalised delta rule needs besides its projections, float [T, H * dk]: the decay
+// w = exp(-dscale * sigmoid(pre + wb)) with pre = sum_j tanh(low[t, j]) up[c, j] (or pre = low[t, c] when up is null),
+// the removal rate a = sigmoid(apre + ab), and per (token, head) kinv = 1 / (sum_head k^2 + 1e-6), the squared length
+// that makes the key a unit vector.  One wave per (token, head).
+template <typename T, typename LT>
+__global__ __launch_bounds__(256) void k_delta_gates(const T* __restrict__ k, int ldk, const LT* __restrict__ low, int ldl,
+                                                     const float* __restrict__ up, int rank,
+                                                     const float* __restrict__ wb, const T* __restrict__ apre, int lda,
+                                                     const float* __restrict__ ab, float* __restrict__ w,
+                                                     float* __restrict__ ar, float* __restrict__ kinv, int nrows,
+                                                     int H, int dk, float dscale) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= nrows) return;
+  const size_t t = row / H;
+  const int hd = row % H;
+  const T* kr = k + t * ldk + hd * dk;
+  float ss = 0.f;
+  for (int c = lane; c < dk; c += 64) {
+    const float v = (float)kr[c];
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  if (lane == 0) kinv[row] = 1.f / (ss + 1e-6f);
+  // the low-rank product: a wave takes tanh of 64 inputs at a time and hands them round; dk <= 256: 4 channels a lane
+  float pre[4] = {0.f, 0.f, 0.f, 0.f};
+  if (up != nullptr) {
+    for (int j0 = 0; j0 < rank; j0 += 64) {
+      const float tl = j0 + lane < rank ? tanhf((float)low[t * ldl + j0 + lane]) : 0.f;
+      const int nj = min(64, rank - j0);
+      for (int jj = 0; jj < nj; ++jj) {
+        const float tj = __shfl(tl, jj, 64);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = lane + 64 * i;
+          if (c < dk) pre[i] += tj * up[(size_t)(hd * dk + c) * rank + j0 + jj];
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = lane + 64 * i;
+    if (c >= dk) break;
+    const int ch = hd * dk + c;
+    float pr = up != nullptr ? pre[i] : (float)low[t * ldl + ch];
+    if (wb != nullptr) pr += wb[ch];
+    float a = (float)apre[t * lda + ch];
+    if (ab != nullptr) a += ab[ch];
+    const size_t o = t * ((size_t)H * dk) + ch;
+    w[o] = expf(-dscale * sigmoidf_(pr));
+    ar[o] = sigmoidf_(a);
+  }
+}
+
+void seq_rope_kv_store(int code, const void* u, int ldu, const float* inv_freq, void* qout, void* kc, void* vc, int nq,
+                       int nk, int nv, int dk, int dims, int half, float mag, int vkeys, int max_len, SeqDesc d,
+                       hipStream_t st) {
+  if (d.Ttot == 0) return;
+  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_rope_kv_store<T>, dim3(d.Ttot), dim3(256), 0, st, (const T*)u, ldu, inv_freq,
+                                          (T*)qout, (T*)kc, (T*)vc, nq, nk, nv, dk, dims, half, mag, vkeys, max_len, d));
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_sigmoid_gate(int code, const void* y, const void* gate, int ldg, void* out, int T_, int C, hipStream_t st) {
+  const size_t n = (size_t)T_ * C;
+  if (n == 0) return;
+  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_sigmoid_gate<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                                          (const T*)y, (const T*)gate, ldg, (T*)out, n, C));
+  LIPA_CHECK_LAUNCH();
+}
+
+// low_f32: the decay's pre-activation (or its low-rank input) is float whatever the activation type
+void seq_delta_gates(int code, int low_f32, const void* k, int ldk, const void* low, int ldl, const float* up, int rank,
+                     const float* wb, const void* apre, int lda, const float* ab, float* w, float* ar, float* kinv, int T_,
+                     int H, int dk, float dscale, hipStream_t st) {
+  const int rows = T_ * H;
+  if (rows == 0) return;
+  SEQ_DISPATCH_T(code, {
+    if (low_f32)
+      hipLaunchKernelGGL((k_delta_gates<T, float>), dim3((rows + 3) / 4), dim3(256), 0, st, (const T*)k, ldk,
+                         (const float*)low, ldl, up, rank, wb, (const T*)apre, lda, ab, w, ar, kinv, rows, H, dk, dscale);
+    else
+      hipLaunchKernelGGL((k_delta_gates<T, T>), dim3((rows + 3) / 4), dim3(256), 0, st, (const T*)k, ldk, (const T*)low,
+                         ldl, up, rank, wb, (const T*)apre, lda, ab, w, ar, kinv, rows, H, dk, dscale);
+  });
+  LIPA_CHECK_LAUNCH();
+}
+
 void seq_embed_sincos(int code, const long* tok, const int* pos, const void* table, const float* inv_freq, float* x,
                       int T_, int W, float scale, hipStream_t st) {
   if (T_ == 0) return;
@@ -503,11 +629,12 @@ void seq_polynorm(int code, const void* z, const float* coef, void* out, int T_,
 }
 
 void seq_head_norm_gate(int code, const float* o, const float* w, int per_head, const void* gate, int ldg,
-                        const float* den, const float* efl, void* out, int T_, int H, int dv, float eps, hipStream_t st) {
+                        const float* den, const float* efl, void* out, int ldo, float scale, int T_, int H, int dv,
+                        float eps, hipStream_t st) {
   const int rows = T_ * H;
   if (rows == 0) return;
   SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_head_norm_gate<T>, dim3((rows + 3) / 4), dim3(256), 0, st, o, w, per_head,
-                                          (const T*)gate, ldg, den, efl, (T*)out, rows, H, dv, eps));
+                                          (const T*)gate, ldg, den, efl, (T*)out, ldo, scale, rows, H, dv, eps));
   LIPA_CHECK_LAUNCH();
 }
 

@@ -366,6 +366,85 @@ __global__ __launch_bounds__(256) void k_delta_scan(const T* __restrict__ q, int
   if (colok) store_rows(Sp, r0, dk, Sr);
 }
 
+// Generalised delta rule.  With the unit key u = k / |k|: S <- diag(w) S - (a * u)(u^T S) + k v^T, both the decay and
+// the removal reading the old S; o = S^T r.  Per column of S that is  e = kinv (k . s);  s <- w * s + k (v - a e)
+// with kinv = 1 / (|k|^2 + 1e-6) per (token, head): one dot product, one update, one dot product per token.
+// w, a float [T, H * dk], kinv float [T, H].  The four staged row arrays live in dynamic shared memory (64 KB at
+// dk > 128).
+template <typename T, int R>
+__global__ __launch_bounds__(256) void k_gdr_scan(const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
+                                                  const T* __restrict__ v, int ldv, const float* __restrict__ w,
+                                                  const float* __restrict__ a, const float* __restrict__ kinv,
+                                                  float* __restrict__ S, float* __restrict__ out, int H, int dk, int dv,
+                                                  SeqDesc d) {
+  constexpr int DKP = KR * R, NC = 256 / R;
+  extern __shared__ __attribute__((aligned(16))) float gdr_smem[];
+  float* sk = gdr_smem;
+  float* sq = sk + CT * DKP;
+  float* sd = sq + CT * DKP;
+  float* sa = sd + CT * DKP;
+  float* sv = sa + CT * DKP;          // [CT * NC]
+  float* sb = sv + CT * NC;           // [CT]
+  const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
+  if (d.live && !d.live[s]) return;
+  const int rg = tid % R, cl = tid / R, col = cb * NC + cl, r0 = rg * KR;
+  const bool colok = col < dv;
+  const int t0 = d.seq_off[s], t1 = d.seq_off[s + 1], p0 = d.pos0[s], slot = d.slots[s];
+  float* Sp = S + (((size_t)slot * H + hd) * dv + (colok ? col : 0)) * dk;
+  float Sr[KR];
+  load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
+  float fk[R], fq[R], fd[R], fa[R], fv[(16 + R - 1) / R], fb = 0.f;
+  auto fetch = [&](int c0) {
+    const int n = min(CT, t1 - c0);
+    fetch_rows<T, R>(fk, k + (size_t)c0 * ldk, ldk, hd * dk, dk, n, 1.f, 0.f);
+    fetch_rows<T, R>(fq, q + (size_t)c0 * ldq, ldq, hd * dk, dk, n, 1.f, 0.f);
+    fetch_rows<float, R>(fd, w + (size_t)c0 * H * dk, (size_t)H * dk, hd * dk, dk, n, 1.f, 1.f);
+    fetch_rows<float, R>(fa, a + (size_t)c0 * H * dk, (size_t)H * dk, hd * dk, dk, n, 1.f, 0.f);
+    fetch_cols<T, R>(fv, v + (size_t)c0 * ldv, ldv, hd * dv, cb, dv, n);
+    if (tid < n) fb = kinv[(size_t)(c0 + tid) * H + hd];
+  };
+  if (t0 < t1) fetch(t0);
+  for (int c0 = t0; c0 < t1; c0 += CT) {
+    const int n = min(CT, t1 - c0);
+    __syncthreads();
+    commit_rows<R>(sk, fk);
+    commit_rows<R>(sq, fq);
+    commit_rows<R>(sd, fd);
+    commit_rows<R>(sa, fa);
+    commit_cols<R>(sv, fv);
+    if (tid < n) sb[tid] = fb;
+    __syncthreads();
+    if (c0 + CT < t1) fetch(c0 + CT);
+    for (int tt = 0; tt < n; ++tt) {
+      f32x4 kk[KR / 4];
+      float dot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i4 = 0; i4 < KR / 4; ++i4) {
+        kk[i4] = *reinterpret_cast<const f32x4*>(sk + tt * DKP + r0 + 4 * i4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dot[j] += Sr[4 * i4 + j] * kk[i4][j];
+      }
+      const float e = sb[tt] * group_sum<R>((dot[0] + dot[1]) + (dot[2] + dot[3]));
+      const float vv = sv[tt * NC + cl];
+      float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i4 = 0; i4 < KR / 4; ++i4) {
+        const f32x4 wd = *reinterpret_cast<const f32x4*>(sd + tt * DKP + r0 + 4 * i4);
+        const f32x4 ar = *reinterpret_cast<const f32x4*>(sa + tt * DKP + r0 + 4 * i4);
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * DKP + r0 + 4 * i4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Sr[4 * i4 + j] = wd[j] * Sr[4 * i4 + j] + kk[i4][j] * (vv - ar[j] * e);
+          o[j] += Sr[4 * i4 + j] * qq[j];
+        }
+      }
+      const float ov = group_sum<R>((o[0] + o[1]) + (o[2] + o[3]));
+      if (rg == 0 && colok) out[((size_t)(c0 + tt) * H + hd) * dv + col] = ov;
+    }
+  }
+  if (colok) store_rows(Sp, r0, dk, Sr);
+}
+
 // State-space duality form of a selective state space (Mamba-2): per head a scalar decay and step size,
 // dt = softplus(dtraw + dt_bias), S <- exp(-exp(A_log) dt) S + B (dt x)^T, y = S^T C + D x.  S is [N, P] per head, held
 // as [P, N] rows like the other recurrences (key size N = dk, value size P = dv); head hd reads B and C of group
@@ -502,6 +581,29 @@ void seq_delta_scan(int code, const void* q, int ldq, const void* k, int ldk, co
     constexpr int NC = 256 / R;
     hipLaunchKernelGGL((k_delta_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
                        (const T*)k, ldk, (const T*)v, ldv, g, bpre, S, out, H, G, dk, dv, d);
+  }));
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_gdr_scan(int code, const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* w,
+                  const float* a, const float* kinv, float* S, float* out, int H, int dk, int dv, SeqDesc d,
+                  hipStream_t st) {
+  if (d.B == 0) return;
+  const int Rr = rows_split(dk);
+  SEQ_DISPATCH_T(code, SEQ_DISPATCH_R(Rr, {
+    constexpr int NC = 256 / R;
+    constexpr size_t smem = sizeof(float) * (4 * CT * KR * R + CT * NC + CT);
+    if (smem > 64 * 1024) {                      // above the default limit of a block: ask for it (dk > 128 only)
+      static bool asked = false;
+      if (!asked) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gdr_scan<T, R>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) fprintf(stderr, "k_gdr_scan: %d bytes of LDS refused: %s\n", (int)smem, hipGetErrorString(e));
+        asked = true;
+      }
+    }
+    hipLaunchKernelGGL((k_gdr_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), smem, st, (const T*)q, ldq,
+                       (const T*)k, ldk, (const T*)v, ldv, w, a, kinv, S, out, H, dk, dv, d);
   }));
   LIPA_CHECK_LAUNCH();
 }

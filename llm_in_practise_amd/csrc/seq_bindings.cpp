@@ -27,7 +27,7 @@ void seq_gated_residual(int, float*, const void*, int, const void*, int, const f
 void seq_dual_norm_mean(int, const void*, const void*, const float*, const float*, void*, int, int, float, hipStream_t);
 void seq_polynorm(int, const void*, const float*, void*, int, int, float, hipStream_t);
 void seq_head_norm_gate(int, const float*, const float*, int, const void*, int, const float*, const float*, void*, int,
-                        int, int, float, hipStream_t);
+                        float, int, int, int, float, hipStream_t);
 void seq_decay_gate(const float*, const float*, const float*, float*, int, int, int, hipStream_t);
 void seq_short_conv(int, int, const void*, int, const float*, const float*, void*, void*, int, int, int, const int*,
                     const float* const*, const float*, SeqDesc, float, hipStream_t);
@@ -40,10 +40,10 @@ void seq_rms_act(int, const void*, int, const float*, void*, int, int, float, hi
 void seq_gate_group_norm(int, const float*, const void*, int, const float*, void*, int, int, int, float, hipStream_t);
 void seq_attn_sweep(int, const void*, int, const void*, int, const void*, int, float*, float*, float*, int, int, int,
                     int, int, int, float, const int*, const int*, int, SeqDesc, hipStream_t);
-void seq_latent_kv_store(int, const void*, int, const float*, const float*, void*, int, int, int, int, float, SeqDesc,
-                         hipStream_t);
+void seq_latent_kv_store(int, const void*, int, const float*, const float*, void*, int, int, int, int, float, int, float,
+                         SeqDesc, hipStream_t);
 void seq_latent_q_assemble(int, const void*, size_t, size_t, const void*, int, int, const float*, void*, int, int, int,
-                           int, SeqDesc, hipStream_t);
+                           int, int, float, SeqDesc, hipStream_t);
 void seq_latent_merge(int, const float*, const float*, const float*, const void*, int, void*, int, int, int, int,
                       hipStream_t);
 void seq_route_grouped(const float*, const float*, int*, float*, int, int, int, int, int, float, int, hipStream_t);
@@ -59,9 +59,16 @@ void seq_hyper_mix_norm(int, int, float*, const void*, int, const float*, const 
                         int, int, int, float, hipStream_t);
 void seq_qk_norm_store(int, const void*, int, const float*, const float*, void*, void*, void*, const void*, const float*,
                        int, int, int, int, float, SeqDesc, hipStream_t);
-void seq_gqa_attention(int, const void*, int, const void*, const void*, float*, float*, float*, const float*, int, int,
-                       int, float, void*, int, int, int, int, int, int, float, const int*, const int*, int, SeqDesc,
-                       hipStream_t);
+void seq_gqa_attention(int, const void*, int, const void*, int, const void*, int, float*, float*, float*, const float*,
+                       int, int, int, int, float, const float*, void*, int, float, int, int, int, int, int, int, float,
+                       const int*, const int*, int, SeqDesc, hipStream_t);
+void seq_rope_kv_store(int, const void*, int, const float*, void*, void*, void*, int, int, int, int, int, int, float, int,
+                       int, SeqDesc, hipStream_t);
+void seq_sigmoid_gate(int, const void*, const void*, int, void*, int, int, hipStream_t);
+void seq_delta_gates(int, int, const void*, int, const void*, int, const float*, int, const float*, const void*, int,
+                     const float*, float*, float*, float*, int, int, int, float, hipStream_t);
+void seq_gdr_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, const float*,
+                  float*, float*, int, int, int, SeqDesc, hipStream_t);
 int seq_hyper_max_streams();
 bool seq_attn_mfma_ok(int, int, int, int);
 void seq_ff_act(int, const void*, void*, int, int, int, float, hipStream_t);
@@ -187,14 +194,21 @@ Tensor polynorm(Tensor z, Tensor coef, double eps) {
 }
 
 // den / efl (optional, float [T, H]): o is divided by max(|den|, efl) + 1e-6 first
-Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps, optional<Tensor> den, optional<Tensor> efl) {
+Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps, optional<Tensor> den, optional<Tensor> efl,
+                      optional<Tensor> out_, double scale) {
   f32c(o, "o");
   TORCH_CHECK(o.dim() == 3, "o: [T, H, dv]");
   const int T = (int)o.size(0), H = (int)o.size(1), dv = (int)o.size(2), code = code_of(gate);
   f32c(w, "w");
   TORCH_CHECK(w.numel() == dv || w.numel() == (int64_t)H * dv, "norm weight: [dv] or [H * dv]");
   rows(gate, T, (int64_t)H * dv, code, "gate");
-  auto out = at::empty({T, (int64_t)H * dv}, gate.options());
+  Tensor out;
+  if (out_ && out_->defined()) {                     // a column slice of a wider matrix
+    out = *out_;
+    rows(out, T, (int64_t)H * dv, code, "out");
+  } else {
+    out = at::empty({T, (int64_t)H * dv}, gate.options());
+  }
   const float* dp = nullptr;
   const float* ep = nullptr;
   if (den && den->defined()) {
@@ -206,7 +220,7 @@ Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps, optional<Tens
     ep = efl->data_ptr<float>();
   }
   seq_head_norm_gate(code, o.data_ptr<float>(), w.data_ptr<float>(), w.numel() != dv, gate.data_ptr(), ld(gate), dp, ep,
-                     out.data_ptr(), T, H, dv, (float)eps, stream());
+                     out.data_ptr(), T == 0 ? H * dv : ld(out), (float)scale, T, H, dv, (float)eps, stream());
   return out;
 }
 
@@ -487,7 +501,7 @@ static void check_freq(const Tensor& f, int64_t dims, int64_t dr) {
 }
 
 void latent_kv_store(Tensor u, Tensor w, Tensor inv_freq, Tensor cache, int64_t dims, double eps,
-                     std::vector<Tensor> desc) {
+                     std::vector<Tensor> desc, bool half, double mag) {
   const int code = code_of(u);
   TORCH_CHECK(u.dim() == 2, "u: [T, kv_rank + rot_dim]");
   const int64_t T = u.size(0), R = w.numel(), dr = u.size(1) - R;
@@ -498,13 +512,16 @@ void latent_kv_store(Tensor u, Tensor w, Tensor inv_freq, Tensor cache, int64_t 
   check_latent_cache(cache, R, dr, code);
   SeqDesc d = desc_of(desc, optional<Tensor>(), T);
   seq_latent_kv_store(code, u.data_ptr(), ld(u), w.data_ptr<float>(), inv_freq.data_ptr<float>(), cache.data_ptr(),
-                      (int)R, (int)dr, (int)dims, (int)cache.size(1), (float)eps, d, stream());
+                      (int)R, (int)dr, (int)dims, (int)cache.size(1), (float)eps, half ? 1 : 0, (float)mag, d, stream());
 }
 
 // qa [H, T, R] (any strides with unit inner stride): the unrotated query parts already multiplied by W_uk;
 // q [T, H * (dn + dr)]; gate [T, H] pre-activations or none.  Returns [T, H, R]: gate * softmax-weighted latents.
+// half / mag: the rotation's layout and magnitude; window > 0 or sinks [H]: the grouped-query sweep (one kv head whose
+// values are the first R columns of its key rows) with a sliding window and a sink score per head, no gate.
 Tensor latent_attention(Tensor qa, Tensor q, Tensor cache, optional<Tensor> gate, Tensor inv_freq, int64_t H, int64_t dn,
-                        int64_t dims, double scale, int64_t nsplit, std::vector<Tensor> desc, std::vector<Tensor> tiles) {
+                        int64_t dims, double scale, int64_t nsplit, std::vector<Tensor> desc, std::vector<Tensor> tiles,
+                        bool half, double mag, int64_t window, optional<Tensor> sinks) {
   const int code = code_of(q);
   const int64_t T = q.size(0);
   TORCH_CHECK(qa.is_cuda() && qa.dim() == 3 && qa.size(0) == H && qa.size(1) == T && (qa.numel() == 0 || qa.stride(2) == 1) &&
@@ -538,10 +555,30 @@ Tensor latent_attention(Tensor qa, Tensor q, Tensor cache, optional<Tensor> gate
   }
   auto fo = q.options().dtype(at::kFloat);
   auto Q = at::empty({T, H * (R + dr)}, q.options());
-  auto pm = at::empty({T, H, nsplit}, fo), pl = at::empty({T, H, nsplit}, fo), pu = at::empty({T, H, nsplit, R}, fo);
   auto out = at::empty({T, H, R}, q.options());
   seq_latent_q_assemble(code, qa.data_ptr(), (size_t)qa.stride(0), (size_t)qa.stride(1), q.data_ptr(), ld(q), (int)dn,
-                        inv_freq.data_ptr<float>(), Q.data_ptr(), (int)H, (int)R, (int)dr, (int)dims, d, stream());
+                        inv_freq.data_ptr<float>(), Q.data_ptr(), (int)H, (int)R, (int)dr, (int)dims, half ? 1 : 0,
+                        (float)mag, d, stream());
+  const bool has_sinks = sinks && sinks->defined();
+  if (window > 0 || has_sinks) {
+    TORCH_CHECK(gp == nullptr && window >= 0, "latent attention: no per-head gate with a window or sinks");
+    const float* sp = nullptr;
+    if (has_sinks) {
+      f32c(*sinks, "sinks");
+      TORCH_CHECK(sinks->numel() == H, "sinks: [H]");
+      sp = sinks->data_ptr<float>();
+    }
+    const bool direct = nsplit == 1 && tseq != nullptr && seq_attn_mfma_ok(code, (int)(H * (R + dr)), (int)(R + dr), (int)R) &&
+                        (R + dr) % 8 == 0;
+    const int64_t np = direct ? 0 : T;
+    auto pm = at::empty({np, H, nsplit}, fo), pl = at::empty({np, H, nsplit}, fo), pu = at::empty({np, H, nsplit, R}, fo);
+    seq_gqa_attention(code, Q.data_ptr(), (int)(H * (R + dr)), cache.data_ptr(), (int)(R + dr), cache.data_ptr(),
+                      (int)(R + dr), pm.data_ptr<float>(), pl.data_ptr<float>(), pu.data_ptr<float>(), nullptr, 0, 0,
+                      (int)window, has_sinks ? 1 : 0, 0.f, sp, out.data_ptr(), (int)(H * R), 1.f, (int)H, 1, (int)(R + dr),
+                      (int)R, (int)cache.size(1), (int)nsplit, (float)scale, tseq, tt0, ntiles, d, stream());
+    return out;
+  }
+  auto pm = at::empty({T, H, nsplit}, fo), pl = at::empty({T, H, nsplit}, fo), pu = at::empty({T, H, nsplit, R}, fo);
   seq_attn_sweep(code, Q.data_ptr(), (int)(H * (R + dr)), cache.data_ptr(), (int)(R + dr), cache.data_ptr(),
                  (int)(R + dr), pm.data_ptr<float>(), pl.data_ptr<float>(), pu.data_ptr<float>(), (int)H, 1,
                  (int)(R + dr), (int)R, (int)cache.size(1), (int)nsplit, (float)scale, tseq, tt0, ntiles, d, stream());
@@ -667,10 +704,11 @@ Tensor moe_combine_sorted(Tensor ys, Tensor pos, Tensor idx, Tensor w, Tensor h,
   return out;
 }
 
-// mode 0: tanh-form GELU of z [T, F]; mode 1: clipped GLU, mode 2: SiLU GLU of z [T, 2F] = [gate | up]
+// mode 0: tanh-form GELU of z [T, F]; mode 1: clipped GLU, mode 2: SiLU GLU, mode 3: tanh-form GELU GLU of
+// z [T, 2F] = [gate | up]
 Tensor ff_act(Tensor z, int64_t mode, double limit) {
   TORCH_CHECK(z.is_cuda() && z.is_contiguous() && z.dim() == 2 &&
-                  (mode == 0 || ((mode == 1 || mode == 2) && z.size(1) % 2 == 0)), "z");
+                  (mode == 0 || (mode >= 1 && mode <= 3 && z.size(1) % 2 == 0)), "z");
   const int64_t T = z.size(0), F = mode == 0 ? z.size(1) : z.size(1) / 2;
   auto out = at::empty({T, F}, z.options());
   seq_ff_act(code_of(z), z.data_ptr(), out.data_ptr(), (int)T, (int)F, (int)mode, (float)limit, stream());
@@ -765,7 +803,8 @@ Tensor qk_norm_store(Tensor u, int64_t nq, int64_t nk, Tensor qw, Tensor kw, Ten
 
 Tensor biased_attention(Tensor q, Tensor kc, Tensor vc, optional<Tensor> bias, int64_t H, int64_t G, double scale,
                         int64_t block, bool sink, double sink_logit, int64_t nsplit, std::vector<Tensor> desc,
-                        std::vector<Tensor> tiles) {
+                        std::vector<Tensor> tiles, int64_t window, optional<Tensor> sinks, optional<Tensor> out_,
+                        double out_scale) {
   const int code = code_of(q);
   TORCH_CHECK(q.dim() == 2 && H >= 1 && G >= 1 && H % G == 0 && q.size(1) % H == 0, "q: [T, H * dk]");
   const int64_t T = q.size(0), dk = q.size(1) / H;
@@ -775,7 +814,13 @@ Tensor biased_attention(Tensor q, Tensor kc, Tensor vc, optional<Tensor> bias, i
                   vc.size(2) % G == 0 && code_of(vc) == code, "value cache: [slots, max_len, G * dv]");
   const int64_t dv = vc.size(2) / G, max_len = kc.size(1);
   TORCH_CHECK(dv >= 1 && dv <= seq_attn_max_cols(), "attention: dv above ", seq_attn_max_cols());
-  TORCH_CHECK(nsplit >= 1 && nsplit <= 1024 && block >= 0, "nsplit, block");
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 1024 && block >= 0 && window >= 0, "nsplit, block, window");
+  const float* sp = nullptr;
+  if (sinks && sinks->defined()) {
+    f32c(*sinks, "sinks");
+    TORCH_CHECK(sink && sinks->numel() == H, "sinks: [H]");
+    sp = sinks->data_ptr<float>();
+  }
   const float* bp = nullptr;
   int nd = 0;
   if (bias && bias->defined()) {
@@ -797,16 +842,123 @@ Tensor biased_attention(Tensor q, Tensor kc, Tensor vc, optional<Tensor> bias, i
     TORCH_CHECK((int64_t)ntiles * 32 >= T && nsplit <= 65535 && H <= 65535, "tiles must cover the tokens");
   }
   auto fo = q.options().dtype(at::kFloat);
+  Tensor out;
+  if (out_ && out_->defined()) {                     // a column slice of a wider matrix
+    out = *out_;
+    rows(out, T, H * dv, code, "out");
+  } else {
+    out = at::empty({T, H * dv}, q.options());
+  }
+  const int ldo = T == 0 ? (int)(H * dv) : ld(out);
+  if (ldo % 4 != 0 || ((uintptr_t)out.data_ptr() & 7) != 0) tseq = nullptr;    // the matrix-core sweep stores 8 bytes
   // one key split on the matrix-core sweep writes the output itself: no partial sums
   const bool direct = nsplit == 1 && tseq != nullptr && seq_attn_mfma_ok(code, ld(q), (int)dk, (int)dv) &&
                       (G * dk) % 8 == 0 && (G * dv) % 8 == 0;
   const int64_t np = direct ? 0 : T;
   auto pm = at::empty({np, H, nsplit}, fo), pl = at::empty({np, H, nsplit}, fo);
   auto pu = at::empty({np, H, nsplit, dv}, fo);
-  auto out = at::empty({T, H * dv}, q.options());
-  seq_gqa_attention(code, q.data_ptr(), ld(q), kc.data_ptr(), vc.data_ptr(), pm.data_ptr<float>(), pl.data_ptr<float>(),
-                    pu.data_ptr<float>(), bp, nd, (int)block, sink ? 1 : 0, (float)sink_logit, out.data_ptr(), (int)H,
-                    (int)G, (int)dk, (int)dv, (int)max_len, (int)nsplit, (float)scale, tseq, tt0, ntiles, d, stream());
+  seq_gqa_attention(code, q.data_ptr(), ld(q), kc.data_ptr(), (int)(G * dk), vc.data_ptr(), (int)(G * dv),
+                    pm.data_ptr<float>(), pl.data_ptr<float>(), pu.data_ptr<float>(), bp, nd, (int)block, (int)window,
+                    sink ? 1 : 0, (float)sink_logit, sp, out.data_ptr(), ldo, (float)out_scale, (int)H, (int)G, (int)dk,
+                    (int)dv, (int)max_len, (int)nsplit, (float)scale, tseq, tt0, ntiles, d, stream());
+  return out;
+}
+
+// u [T, nq + nk (+ nv)]: rotated q returned, rotated k and the values (u's v columns, or the k columns as they came) go
+// to the caches at each token's (slot, position)
+Tensor rope_kv_store(Tensor u, int64_t nq, int64_t nk, int64_t H, int64_t G, Tensor inv_freq, int64_t dims, Tensor kc,
+                     Tensor vc, std::vector<Tensor> desc, bool half, double mag, bool values_are_keys) {
+  const int code = code_of(u);
+  TORCH_CHECK(u.dim() == 2 && H >= 1 && G >= 1 && nq % H == 0 && nk % G == 0 && nq / H == nk / G &&
+                  u.size(1) >= nq + nk, "u: [T, H * dk + G * dk (+ nv)]");
+  const int64_t T = u.size(0), nv = values_are_keys ? nk : u.size(1) - nq - nk, dk = nq / H;
+  TORCH_CHECK(nv >= 1, "no value columns");
+  rows(u, T, u.size(1), code, "u");
+  check_freq(inv_freq, dims, dk);
+  check_kv_cache(kc, nk, code, "key cache");
+  check_kv_cache(vc, nv, code, "value cache");
+  TORCH_CHECK(vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "caches: one pool of slots");
+  SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  auto q = at::empty({T, nq}, u.options());
+  seq_rope_kv_store(code, u.data_ptr(), ld(u), inv_freq.data_ptr<float>(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                    (int)nq, (int)nk, (int)nv, (int)dk, (int)dims, half ? 1 : 0, (float)mag, values_are_keys ? 1 : 0,
+                    (int)kc.size(1), d, stream());
+  return q;
+}
+
+Tensor sigmoid_gate(Tensor y, Tensor gate) {
+  const int code = code_of(y);
+  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.dim() == 2, "y: [T, C], contiguous");
+  const int64_t T = y.size(0), C = y.size(1);
+  rows(gate, T, C, code, "gate");
+  auto out = at::empty_like(y);
+  seq_sigmoid_gate(code, y.data_ptr(), gate.data_ptr(), T == 0 ? (int)C : ld(gate), out.data_ptr(), (int)T, (int)C, stream());
+  return out;
+}
+
+// returns {w, a} float [T, H * dk] and kinv float [T, H]
+std::vector<Tensor> delta_rule_gates(Tensor k, Tensor low, optional<Tensor> up, optional<Tensor> wb, Tensor apre,
+                                     optional<Tensor> ab, int64_t H, double dscale) {
+  const int code = code_of(k);
+  TORCH_CHECK(k.dim() == 2 && H >= 1 && k.size(1) % H == 0, "k: [T, H * dk]");
+  const int64_t T = k.size(0), C = k.size(1), dk = C / H;
+  TORCH_CHECK(dk <= seq_scan_max_dk(), "key size above ", seq_scan_max_dk());
+  rows(k, T, C, code, "k");
+  rows(apre, T, C, code, "a_pre");
+  const float* upp = nullptr;
+  int64_t rank = 0;
+  const int low_f32 = low.scalar_type() == at::kFloat;
+  if (up && up->defined()) {
+    f32c(*up, "w_up");
+    TORCH_CHECK(up->dim() == 2 && up->size(0) == C, "w_up: [H * dk, rank]");
+    rank = up->size(1);
+    upp = up->data_ptr<float>();
+    rows(low, T, rank, low_f32 ? 1 : code, "w_low");
+  } else {
+    rows(low, T, C, low_f32 ? 1 : code, "w_pre");
+  }
+  const float* wbp = nullptr;
+  const float* abp = nullptr;
+  if (wb && wb->defined()) {
+    f32c(*wb, "w_bias");
+    TORCH_CHECK(wb->numel() == C, "w_bias: [H * dk]");
+    wbp = wb->data_ptr<float>();
+  }
+  if (ab && ab->defined()) {
+    f32c(*ab, "a_bias");
+    TORCH_CHECK(ab->numel() == C, "a_bias: [H * dk]");
+    abp = ab->data_ptr<float>();
+  }
+  auto fo = k.options().dtype(at::kFloat);
+  auto w = at::empty({T, C}, fo), a = at::empty({T, C}, fo), kinv = at::empty({T, H}, fo);
+  seq_delta_gates(code, low_f32, k.data_ptr(), T == 0 ? (int)C : ld(k), low.data_ptr(), T == 0 ? 1 : ld(low), upp,
+                  (int)rank, wbp, apre.data_ptr(), T == 0 ? (int)C : ld(apre), abp, w.data_ptr<float>(),
+                  a.data_ptr<float>(), kinv.data_ptr<float>(), (int)T, (int)H, (int)dk, (float)dscale, stream());
+  return {w, a, kinv};
+}
+
+// r, k [T, H * dk], v [T, H * dv]; w, a float [T, H * dk], kinv float [T, H]; S float [slots, H, dv, dk] in place
+Tensor general_delta_scan(Tensor r, Tensor k, Tensor v, Tensor w, Tensor a, Tensor kinv, Tensor S, int64_t H,
+                          std::vector<Tensor> desc, optional<Tensor> live) {
+  const int code = code_of(r);
+  const int64_t T = r.size(0);
+  TORCH_CHECK(H >= 1 && r.dim() == 2 && r.size(1) % H == 0 && v.dim() == 2 && v.size(1) % H == 0,
+              "r/k: [T, H * dk], v: [T, H * dv]");
+  const int64_t dk = r.size(1) / H, dv = v.size(1) / H;
+  rows(r, T, H * dk, code, "r");
+  rows(k, T, H * dk, code, "k");
+  rows(v, T, H * dv, code, "v");
+  f32c(w, "w");
+  f32c(a, "a");
+  f32c(kinv, "kinv");
+  TORCH_CHECK(w.numel() == T * H * dk && a.numel() == T * H * dk && kinv.numel() == T * H, "w, a: [T, H * dk], kinv: [T, H]");
+  TORCH_CHECK(dk <= seq_scan_max_dk(), "key size above ", seq_scan_max_dk());
+  check_state(S, H, dv, dk);
+  SeqDesc d = desc_of(desc, live, T);
+  auto out = at::empty({T, H, dv}, S.options());
+  seq_gdr_scan(code, r.data_ptr(), ld(r), k.data_ptr(), ld(k), v.data_ptr(), ld(v), w.data_ptr<float>(),
+               a.data_ptr<float>(), kinv.data_ptr<float>(), S.data_ptr<float>(), out.data_ptr<float>(), (int)H, (int)dk,
+               (int)dv, d, stream());
   return out;
 }
 
@@ -840,4 +992,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("hyper_mix_norm", &hyper_mix_norm);
   m.def("qk_norm_store", &qk_norm_store);
   m.def("biased_attention", &biased_attention);
+  m.def("rope_kv_store", &rope_kv_store);
+  m.def("sigmoid_gate", &sigmoid_gate);
+  m.def("delta_rule_gates", &delta_rule_gates);
+  m.def("general_delta_scan", &general_delta_scan);
 }

@@ -262,10 +262,10 @@ class ParallelWindowDeltaMixer(_Sublayer):
                           sb, True, self.mag, True)
         biased_attention(q, st["k"], st["v"], None, self.H, self.G, self.scale, sb, 0, None,
                          _window_splits(sb.cache, self.window) if sb.decode else 1, self.window, both[:, :self.nq], self.ls)
-        # right: decays, unit keys and removal vectors in float, then the scan over the slot's matrix
-        w, u, au = delta_rule_gates(P[:, o[3]:o[4]], P[:, o[7]:o[8]], self.w_up, self.w0, P[:, o[6]:o[7]], None, self.HR,
+        # right: decays, removal rates and key lengths in float, then the scan over the slot's matrix
+        w, a, kinv = delta_rule_gates(P[:, o[3]:o[4]], P[:, o[7]:o[8]], self.w_up, self.w0, P[:, o[6]:o[7]], None, self.HR,
                                     DECAY_SCALE)
-        s = general_delta_scan(P[:, o[2]:o[3]], P[:, o[3]:o[4]], P[:, o[4]:o[5]], w, u, au, st["S"], self.HR, sb)
+        s = general_delta_scan(P[:, o[2]:o[3]], P[:, o[3]:o[4]], P[:, o[4]:o[5]], w, a, kinv, st["S"], self.HR, sb)
         head_norm_gate(s, self.norm, P[:, o[5]:o[6]], eps, None, None, both[:, self.nq:], self.rs)
         return both @ self.w_o.t()
 

@@ -60,22 +60,24 @@ def ssd_scan(c, b, x, dt_raw, dt_bias, a_log, d_skip, S, heads: int, groups: int
 
 
 def delta_rule_gates(k, w_low, w_up, w_bias, a_pre, a_bias, heads: int, decay_scale: float):
-    """What :func:`general_delta_scan` needs besides the projections, all float ``[T, H*dk]``: the decay
-    ``w = exp(-decay_scale * sigmoid(w_pre + w_bias))``, the unit key ``u = k / sqrt(sum_head(k^2) + 1e-6)`` and
-    ``a * u`` with the removal rate ``a = sigmoid(a_pre + a_bias)``.  The decay's pre-activation is low-rank:
-    ``w_pre = tanh(w_low) w_up^T`` with ``w_low`` ``[T, r]`` (the down-projection's output) and ``w_up`` float
-    ``[H*dk, r]``, evaluated in float here; ``w_up = None``: ``w_low`` is ``w_pre`` itself ``[T, H*dk]``.
-    ``k`` / ``a_pre`` ``[T, H*dk]`` in the activation dtype (column slices are fine); biases float ``[H*dk]`` or None."""
+    """What :func:`general_delta_scan` needs besides the projections, all float: the decay
+    ``w = exp(-decay_scale * sigmoid(w_pre + w_bias))`` and the removal rate ``a = sigmoid(a_pre + a_bias)``, both
+    ``[T, H*dk]``, and ``kinv = 1 / (sum_head(k^2) + 1e-6)`` ``[T, H]`` (the squared length that makes the key a unit
+    vector).  The decay's pre-activation is low-rank: ``w_pre = tanh(w_low) w_up^T`` with ``w_low`` ``[T, r]`` (the
+    down-projection's output) and ``w_up`` float ``[H*dk, r]``, evaluated in float here; ``w_up = None``: ``w_low`` is
+    ``w_pre`` itself ``[T, H*dk]``.  ``k`` / ``a_pre`` ``[T, H*dk]`` in the activation dtype (column slices are fine);
+    biases float ``[H*dk]`` or None."""
     if use_seq(k):
         return tuple(native_seq().delta_rule_gates(k, w_low, w_up, w_bias, a_pre, a_bias, heads, decay_scale))
     return ref.delta_rule_gates(k, w_low, w_up, w_bias, a_pre, a_bias, heads, decay_scale)
 
 
-def general_delta_scan(r, k, v, w, u, au, S, heads: int, sb):
-    """Per head, with ``S`` ``[dk, dv]``: ``S <- diag(w) S - au (u^T S) + k v^T`` (decay and removal both read the old
-    ``S``), ``o = S^T r``.  ``r, k`` ``[T, H*dk]``, ``v`` ``[T, H*dv]`` in the activation dtype; ``w, u, au`` float
-    ``[T, H*dk]`` (:func:`delta_rule_gates`); ``S`` float ``[slots, H, dv, dk]`` in place.  Returns float
-    ``[T, H, dv]``."""
+def general_delta_scan(r, k, v, w, a, kinv, S, heads: int, sb):
+    """Per head, with ``S`` ``[dk, dv]`` and the unit key ``u = k sqrt(kinv)``: ``S <- diag(w) S - (a * u)(u^T S) + k v^T``
+    (decay and removal both read the old ``S``), ``o = S^T r``; evaluated as
+    ``S <- diag(w) S + k (v - a * e)^T`` per key channel with ``e = kinv (k^T S)``.  ``r, k`` ``[T, H*dk]``, ``v``
+    ``[T, H*dv]`` in the activation dtype; ``w, a`` float ``[T, H*dk]``, ``kinv`` float ``[T, H]``
+    (:func:`delta_rule_gates`); ``S`` float ``[slots, H, dv, dk]`` in place.  Returns float ``[T, H, dv]``."""
     if use_seq(r):
-        return native_seq().general_delta_scan(r, k, v, w, u, au, S, heads, sb.desc, sb.live)
-    return ref.general_delta_scan(r, k, v, w, u, au, S, heads, sb)
+        return native_seq().general_delta_scan(r, k, v, w, a, kinv, S, heads, sb.desc, sb.live)
+    return ref.general_delta_scan(r, k, v, w, a, kinv, S, heads, sb)

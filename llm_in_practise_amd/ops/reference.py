@@ -553,16 +553,15 @@ def delta_rule_gates(k, w_low, w_up, w_bias, a_pre, a_bias, H: int, decay_scale:
     w_pre = w_low.float() if w_up is None else torch.tanh(w_low.float()) @ w_up.float().t()
     w = torch.exp(-decay_scale * torch.sigmoid(w_pre + (w_bias if w_bias is not None else 0.0)))
     a = torch.sigmoid(a_pre.float() + (a_bias if a_bias is not None else 0.0))
-    kf = k.float().view(T, H, dk)
-    u = (kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + 1e-6)).reshape(T, H * dk)
-    return w.contiguous(), u.contiguous(), (a * u).contiguous()
+    kinv = 1.0 / (k.float().view(T, H, dk).pow(2).sum(-1) + 1e-6)
+    return w.contiguous(), a.contiguous(), kinv.contiguous()
 
 
-def general_delta_scan(r, k, v, w, u, au, S, H: int, sb):
+def general_delta_scan(r, k, v, w, a, kinv, S, H: int, sb):
     T = r.shape[0]
     dk, dv = r.shape[1] // H, v.shape[1] // H
     rf, kf, vf = r.float().view(T, H, dk), k.float().view(T, H, dk), v.float().view(T, H, dv)
-    wf, uf, af = w.view(T, H, dk), u.view(T, H, dk), au.view(T, H, dk)
+    wf, af = w.view(T, H, dk), a.view(T, H, dk)
     out = torch.empty(T, H, dv, dtype=torch.float32, device=r.device)
     off, slots, pos0 = sb.host()
     for b, slot in enumerate(slots):
@@ -570,8 +569,8 @@ def general_delta_scan(r, k, v, w, u, au, S, H: int, sb):
             continue
         s = torch.zeros_like(S[slot]) if pos0[b] == 0 else S[slot].clone()   # [H, dv, dk]
         for t in range(off[b], off[b + 1]):
-            d = (s * uf[t][:, None, :]).sum(-1)                              # [H, dv]: u^T S of the old state
-            s = s * wf[t][:, None, :] - d[:, :, None] * af[t][:, None, :] + vf[t][:, :, None] * kf[t][:, None, :]
+            e = (s * kf[t][:, None, :]).sum(-1) * kinv[t][:, None]           # [H, dv]: (k^T S) / |k|^2 of the old state
+            s = s * wf[t][:, None, :] + kf[t][:, None, :] * (vf[t][:, :, None] - af[t][:, None, :] * e[:, :, None])
             out[t] = (s * rf[t][:, None, :]).sum(-1)
         S[slot] = s
     return out
