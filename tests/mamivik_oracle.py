@@ -163,7 +163,9 @@ def forward(cfg: dict, W: dict, tokens):
     after = []
     for i, lc in enumerate(cfg["layers"]):
         p = f"l{i}."
-        h = input_conv(unit_rms(x, eps) * W[p + "norm1"].to(F64), W[p + "canon1"].to(F64))
+        h = unit_rms(x, eps) * W[p + "norm1"].to(F64)
+        if p + "canon1" in W:
+            h = input_conv(h, W[p + "canon1"].to(F64))
         if lc["type"] == "latent_attention":
             x = x + latent_attention(W, p + "mix.", lc["mixer"], h, eps)
         else:
