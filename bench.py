@@ -224,14 +224,15 @@ def main():
                     help="time budget of each sub-record (host / faithful / selective / zero3); past it the headline "
                          "line is printed with '<record>': {'error': ...} and the process exits 0 "
                          "(default: 240 s, 420 s for the zero3 sub-record, which builds its own model)")
-    ap.add_argument("--workload", default="train", choices=["train", "hybrid-serve", "dogudra-serve", "kitonex-serve"],
+    ap.add_argument("--workload", default="train", choices=["train", "hybrid-serve", "dogudra-serve", "kitonex-serve", "mamivik-serve"],
                     help="train (default): the headline fine-tuning step.  hybrid-serve: prefill / decode tokens/s of "
                          "the Mobupel hybrid beside Qwen3 at equal size through the serving engine (one GPU); "
                          "dogudra-serve: the same for the Dogudra design beside Mobupel and Qwen3; "
                          "kitonex-serve: the same for the Kitonex design beside Dogudra and Qwen3; "
+                         "mamivik-serve: the same for the Mamivik design beside Mobupel and Qwen3; "
                          "--sizes / --serve-batch / --serve-prompt / --serve-decode-steps shape both")
     ap.add_argument("--serve-models", default=None,
-                    help="dogudra-serve / kitonex-serve: which of the three models to time (default: all)")
+                    help="dogudra-serve / kitonex-serve / mamivik-serve: which of the three models to time (default: all)")
     ap.add_argument("--sizes", default="w1024,w2048")
     ap.add_argument("--serve-batch", type=int, default=8)
     ap.add_argument("--serve-prompt", type=int, default=1024)
@@ -253,6 +254,12 @@ def main():
         print(json.dumps(kitonex_run(tuple(args.sizes.split(",")), args.serve_batch, args.serve_prompt,
                                      args.serve_decode_steps,
                                      models=tuple((args.serve_models or "kitonex,dogudra,qwen3").split(",")))), flush=True)
+        return
+    if args.workload == "mamivik-serve":
+        from llm_in_practise_amd.bench.mamivik_serve import run as mamivik_run
+        print(json.dumps(mamivik_run(tuple(args.sizes.split(",")), args.serve_batch, args.serve_prompt,
+                                     args.serve_decode_steps,
+                                     models=tuple((args.serve_models or "mamivik,mobupel,qwen3").split(",")))), flush=True)
         return
     from llm_in_practise_amd.ops import gemm as _lin
     if args.nf4_gemm is not None:        # else the LIPA_NF4_GEMM environment choice stands
