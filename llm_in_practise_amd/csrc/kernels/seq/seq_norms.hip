@@ -506,54 +506,73 @@ __global__ __launch_bounds__(256) void k_sigmoid_gate(const T* __restrict__ y, c
 // What the generalised delta rule needs besides its projections, float [T, H * dk]: the decay
 // w = exp(-dscale * sigmoid(pre + wb)) with pre = sum_j tanh(low[t, j]) up[c, j] (or pre = low[t, c] when up is null),
 // the removal rate a = sigmoid(apre + ab), and per (token, head) kinv = 1 / (sum_head k^2 + 1e-6), the squared length
-// that makes the key a unit vector.  One wave per (token, head).
-template <typename T, typename LT>
+// that makes the key a unit vector.  One wave per (head, tpw consecutive tokens): a lane keeps the low-rank rows of
+// its channels in registers (RK = 16: rank <= 16) and takes tanh of one low-rank input per token, handed round the
+// wave; dk <= 256: 4 channels a lane.
+template <typename T, typename LT, int RK>
 __global__ __launch_bounds__(256) void k_delta_gates(const T* __restrict__ k, int ldk, const LT* __restrict__ low, int ldl,
                                                      const float* __restrict__ up, int rank,
                                                      const float* __restrict__ wb, const T* __restrict__ apre, int lda,
                                                      const float* __restrict__ ab, float* __restrict__ w,
-                                                     float* __restrict__ ar, float* __restrict__ kinv, int nrows,
-                                                     int H, int dk, float dscale) {
+                                                     float* __restrict__ ar, float* __restrict__ kinv, int T_, int tpw,
+                                                     int nrows, int H, int dk, float dscale) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= nrows) return;
-  const size_t t = row / H;
-  const int hd = row % H;
-  const T* kr = k + t * ldk + hd * dk;
-  float ss = 0.f;
-  for (int c = lane; c < dk; c += 64) {
-    const float v = (float)kr[c];
-    ss += v * v;
-  }
-  ss = wave_sum(ss);
-  if (lane == 0) kinv[row] = 1.f / (ss + 1e-6f);
-  // the low-rank product: a wave takes tanh of 64 inputs at a time and hands them round; dk <= 256: 4 channels a lane
-  float pre[4] = {0.f, 0.f, 0.f, 0.f};
-  if (up != nullptr) {
-    for (int j0 = 0; j0 < rank; j0 += 64) {
-      const float tl = j0 + lane < rank ? tanhf((float)low[t * ldl + j0 + lane]) : 0.f;
-      const int nj = min(64, rank - j0);
-      for (int jj = 0; jj < nj; ++jj) {
-        const float tj = __shfl(tl, jj, 64);
+  const int hd = row % H, t0 = (row / H) * tpw, t1 = min(T_, t0 + tpw);
+  float upr[4][RK > 0 ? RK : 1], bw[4], ba[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int c = lane + 64 * i;
-          if (c < dk) pre[i] += tj * up[(size_t)(hd * dk + c) * rank + j0 + jj];
+  for (int i = 0; i < 4; ++i) {
+    const int c = lane + 64 * i, ch = hd * dk + c;
+    bw[i] = (c < dk && wb != nullptr) ? wb[ch] : 0.f;
+    ba[i] = (c < dk && ab != nullptr) ? ab[ch] : 0.f;
+    if (RK > 0)
+#pragma unroll
+      for (int j = 0; j < RK; ++j) upr[i][j] = (c < dk && j < rank) ? up[(size_t)ch * rank + j] : 0.f;
+  }
+  for (int t = t0; t < t1; ++t) {
+    const T* kr = k + (size_t)t * ldk + hd * dk;
+    float ss = 0.f;
+    for (int c = lane; c < dk; c += 64) {
+      const float v = (float)kr[c];
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) kinv[(size_t)t * H + hd] = 1.f / (ss + 1e-6f);
+    float pre[4] = {0.f, 0.f, 0.f, 0.f};
+    if (up != nullptr) {
+      for (int j0 = 0; j0 < rank; j0 += 64) {
+        const float tl = j0 + lane < rank ? tanhf((float)low[(size_t)t * ldl + j0 + lane]) : 0.f;
+        if (RK > 0) {
+#pragma unroll
+          for (int jj = 0; jj < RK; ++jj) {
+            const float tj = __shfl(tl, jj, 64);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pre[i] += tj * upr[i][jj];
+          }
+        } else {
+          const int nj = min(64, rank - j0);
+          for (int jj = 0; jj < nj; ++jj) {
+            const float tj = __shfl(tl, jj, 64);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int c = lane + 64 * i;
+              if (c < dk) pre[i] += tj * up[(size_t)(hd * dk + c) * rank + j0 + jj];
+            }
+          }
         }
       }
     }
-  }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = lane + 64 * i;
-    if (c >= dk) break;
-    const int ch = hd * dk + c;
-    float pr = up != nullptr ? pre[i] : (float)low[t * ldl + ch];
-    if (wb != nullptr) pr += wb[ch];
-    float a = (float)apre[t * lda + ch];
-    if (ab != nullptr) a += ab[ch];
-    const size_t o = t * ((size_t)H * dk) + ch;
-    w[o] = expf(-dscale * sigmoidf_(pr));
-    ar[o] = sigmoidf_(a);
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c >= dk) break;
+      const int ch = hd * dk + c;
+      const float pr = (up != nullptr ? pre[i] : (float)low[(size_t)t * ldl + ch]) + bw[i];
+      const float a = (float)apre[(size_t)t * lda + ch] + ba[i];
+      const size_t o = (size_t)t * ((size_t)H * dk) + ch;
+      w[o] = expf(-dscale * sigmoidf_(pr));
+      ar[o] = sigmoidf_(a);
+    }
   }
 }
 
@@ -578,16 +597,21 @@ void seq_sigmoid_gate(int code, const void* y, const void* gate, int ldg, void* 
 void seq_delta_gates(int code, int low_f32, const void* k, int ldk, const void* low, int ldl, const float* up, int rank,
                      const float* wb, const void* apre, int lda, const float* ab, float* w, float* ar, float* kinv, int T_,
                      int H, int dk, float dscale, hipStream_t st) {
-  const int rows = T_ * H;
-  if (rows == 0) return;
+  if (T_ == 0) return;
+  const int tpw = T_ >= 256 ? 8 : 1;                 // long steps: a wave keeps its low-rank rows for 8 tokens
+  const int rows = ((T_ + tpw - 1) / tpw) * H;
+  const bool reg = up != nullptr && rank <= 16;
+#define SEQ_GATES_LAUNCH(LT, RK)                                                                                       \
+  hipLaunchKernelGGL((k_delta_gates<T, LT, RK>), dim3((rows + 3) / 4), dim3(256), 0, st, (const T*)k, ldk, (const LT*)low, \
+                     ldl, up, rank, wb, (const T*)apre, lda, ab, w, ar, kinv, T_, tpw, rows, H, dk, dscale)
   SEQ_DISPATCH_T(code, {
-    if (low_f32)
-      hipLaunchKernelGGL((k_delta_gates<T, float>), dim3((rows + 3) / 4), dim3(256), 0, st, (const T*)k, ldk,
-                         (const float*)low, ldl, up, rank, wb, (const T*)apre, lda, ab, w, ar, kinv, rows, H, dk, dscale);
-    else
-      hipLaunchKernelGGL((k_delta_gates<T, T>), dim3((rows + 3) / 4), dim3(256), 0, st, (const T*)k, ldk, (const T*)low,
-                         ldl, up, rank, wb, (const T*)apre, lda, ab, w, ar, kinv, rows, H, dk, dscale);
+    if (low_f32) {
+      if (reg) SEQ_GATES_LAUNCH(float, 16); else SEQ_GATES_LAUNCH(float, 0);
+    } else {
+      if (reg) SEQ_GATES_LAUNCH(T, 16); else SEQ_GATES_LAUNCH(T, 0);
+    }
   });
+#undef SEQ_GATES_LAUNCH
   LIPA_CHECK_LAUNCH();
 }
 

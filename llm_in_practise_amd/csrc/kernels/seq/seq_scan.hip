@@ -369,25 +369,38 @@ __global__ __launch_bounds__(256) void k_delta_scan(const T* __restrict__ q, int
 // Generalised delta rule.  With the unit key u = k / |k|: S <- diag(w) S - (a * u)(u^T S) + k v^T, both the decay and
 // the removal reading the old S; o = S^T r.  Per column of S that is  e = kinv (k . s);  s <- w * s + k (v - a e)
 // with kinv = 1 / (|k|^2 + 1e-6) per (token, head): one dot product, one update, one dot product per token.
-// w, a float [T, H * dk], kinv float [T, H].  The four staged row arrays live in dynamic shared memory (64 KB at
+// w, a float [T, H * dk], kinv float [T, H].  The four staged row arrays live in dynamic shared memory (81 KB at
 // dk > 128).
+// commit_rows with 4 floats of padding after every lane's 16 rows: the 16-byte reads of lanes rg and rg + 4 then fall
+// into different banks (unpadded, their rows are 256 bytes apart: the same banks)
+constexpr int KRP = KR + 4;
+template <int R>
+__device__ __forceinline__ void commit_rows_padded(float* dst, const float (&v)[R]) {
+  constexpr int DKP = KR * R;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int e = threadIdx.x + 256 * i, tt = e / DKP, r = e % DKP;
+    dst[tt * (KRP * R) + (r / KR) * KRP + (r % KR)] = v[i];
+  }
+}
+
 template <typename T, int R>
 __global__ __launch_bounds__(256) void k_gdr_scan(const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
                                                   const T* __restrict__ v, int ldv, const float* __restrict__ w,
                                                   const float* __restrict__ a, const float* __restrict__ kinv,
                                                   float* __restrict__ S, float* __restrict__ out, int H, int dk, int dv,
                                                   SeqDesc d) {
-  constexpr int DKP = KR * R, NC = 256 / R;
+  constexpr int DKP = KR * R, NC = 256 / R, LDR = KRP * R;       // LDR: floats of a staged token row, padded
   extern __shared__ __attribute__((aligned(16))) float gdr_smem[];
   float* sk = gdr_smem;
-  float* sq = sk + CT * DKP;
-  float* sd = sq + CT * DKP;
-  float* sa = sd + CT * DKP;
-  float* sv = sa + CT * DKP;          // [CT * NC]
+  float* sq = sk + CT * LDR;
+  float* sd = sq + CT * LDR;
+  float* sa = sd + CT * LDR;
+  float* sv = sa + CT * LDR;          // [CT * NC]
   float* sb = sv + CT * NC;           // [CT]
   const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
   if (d.live && !d.live[s]) return;
-  const int rg = tid % R, cl = tid / R, col = cb * NC + cl, r0 = rg * KR;
+  const int rg = tid % R, cl = tid / R, col = cb * NC + cl, r0 = rg * KR, l0 = rg * KRP;
   const bool colok = col < dv;
   const int t0 = d.seq_off[s], t1 = d.seq_off[s + 1], p0 = d.pos0[s], slot = d.slots[s];
   float* Sp = S + (((size_t)slot * H + hd) * dv + (colok ? col : 0)) * dk;
@@ -407,35 +420,46 @@ __global__ __launch_bounds__(256) void k_gdr_scan(const T* __restrict__ q, int l
   for (int c0 = t0; c0 < t1; c0 += CT) {
     const int n = min(CT, t1 - c0);
     __syncthreads();
-    commit_rows<R>(sk, fk);
-    commit_rows<R>(sq, fq);
-    commit_rows<R>(sd, fd);
-    commit_rows<R>(sa, fa);
+#pragma unroll
+    for (int i = 0; i < R; ++i) fa[i] *= fk[i];          // staged as k * a: the update is then two fused steps
+    commit_rows_padded<R>(sk, fk);
+    commit_rows_padded<R>(sq, fq);
+    commit_rows_padded<R>(sd, fd);
+    commit_rows_padded<R>(sa, fa);
     commit_cols<R>(sv, fv);
     if (tid < n) sb[tid] = fb;
     __syncthreads();
     if (c0 + CT < t1) fetch(c0 + CT);
+    // the dot product k . s of a token runs in the same sweep as the read-out of the token before it (both read the
+    // new s), so only the chunk's first token needs a sweep of its own.  Every row vector is read from LDS where it
+    // is used (no register copies from token to token: the scan is bound by its vector instructions).
+    float dot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i4 = 0; i4 < KR / 4; ++i4) {
+      const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + l0 + 4 * i4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dot[j] += Sr[4 * i4 + j] * kk[j];
+    }
     for (int tt = 0; tt < n; ++tt) {
-      f32x4 kk[KR / 4];
-      float dot[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int i4 = 0; i4 < KR / 4; ++i4) {
-        kk[i4] = *reinterpret_cast<const f32x4*>(sk + tt * DKP + r0 + 4 * i4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dot[j] += Sr[4 * i4 + j] * kk[i4][j];
-      }
+      const int tn = min(tt + 1, n - 1);
       const float e = sb[tt] * group_sum<R>((dot[0] + dot[1]) + (dot[2] + dot[3]));
       const float vv = sv[tt * NC + cl];
       float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
+      for (int j = 0; j < 4; ++j) dot[j] = 0.f;
+#pragma unroll
       for (int i4 = 0; i4 < KR / 4; ++i4) {
-        const f32x4 wd = *reinterpret_cast<const f32x4*>(sd + tt * DKP + r0 + 4 * i4);
-        const f32x4 ar = *reinterpret_cast<const f32x4*>(sa + tt * DKP + r0 + 4 * i4);
-        const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * DKP + r0 + 4 * i4);
+        const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + tt * LDR + l0 + 4 * i4);
+        const f32x4 wd = *reinterpret_cast<const f32x4*>(sd + tt * LDR + l0 + 4 * i4);
+        const f32x4 ka = *reinterpret_cast<const f32x4*>(sa + tt * LDR + l0 + 4 * i4);
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * LDR + l0 + 4 * i4);
+        const f32x4 kn = *reinterpret_cast<const f32x4*>(sk + tn * LDR + l0 + 4 * i4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          Sr[4 * i4 + j] = wd[j] * Sr[4 * i4 + j] + kk[i4][j] * (vv - ar[j] * e);
-          o[j] += Sr[4 * i4 + j] * qq[j];
+          const float sn = (wd[j] * Sr[4 * i4 + j] + kk[j] * vv) - ka[j] * e;
+          Sr[4 * i4 + j] = sn;
+          o[j] += sn * qq[j];
+          dot[j] += sn * kn[j];
         }
       }
       const float ov = group_sum<R>((o[0] + o[1]) + (o[2] + o[3]));
@@ -592,7 +616,7 @@ void seq_gdr_scan(int code, const void* q, int ldq, const void* k, int ldk, cons
   const int Rr = rows_split(dk);
   SEQ_DISPATCH_T(code, SEQ_DISPATCH_R(Rr, {
     constexpr int NC = 256 / R;
-    constexpr size_t smem = sizeof(float) * (4 * CT * KR * R + CT * NC + CT);
+    constexpr size_t smem = sizeof(float) * (4 * CT * KRP * R + CT * NC + CT);
     if (smem > 64 * 1024) {                      // above the default limit of a block: ask for it (dk > 128 only)
       static bool asked = false;
       if (!asked) {
