@@ -119,7 +119,8 @@ def _check_rot(rot: dict | None, width: int):
 
 
 def tensor_shapes(cfg: MamivikConfig, decay_rank: int = 16) -> dict[str, tuple]:
-    """Every checkpoint tensor of a config and its shape.  The decay's rank is a tensor's shape, not a config entry."""
+    """Every checkpoint tensor of a config and its shape.  The decay's rank is a tensor's shape, not a config entry;
+    a query rank that the config leaves out reads as 0 (the loader takes it from the tensor)."""
     Wd = cfg.width
     out = {"embed": (cfg.vocab, Wd), "final.norm": (), "head": (cfg.vocab, Wd)}
     for i, lc in enumerate(cfg.layers):
@@ -128,7 +129,7 @@ def tensor_shapes(cfg: MamivikConfig, decay_rank: int = 16) -> dict[str, tuple]:
         if cfg.taps:
             out[p + "canon1"] = (Wd, cfg.taps)
         if lc["type"] == "latent_attention":
-            H, dn, dr, dv, R, qr = (int(m[k]) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank", "q_rank"))
+            H, dn, dr, dv, R, qr = (int(m.get(k, 0)) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank", "q_rank"))
             out.update({q + "dq": (qr, Wd), q + "dq.norm": (qr,), q + "uq": (H * (dn + dr), qr),
                         q + "dkv": (R + dr, Wd), q + "dkv.norm": (R,), q + "uk": (H * dn, R), q + "uv": (H * dv, R),
                         q + "sink": (H,), q + "g": (H * dv, Wd), q + "o": (Wd, H * dv)})
@@ -174,10 +175,11 @@ def random_weights(cfg: MamivikConfig, seed: int = 0, decay_rank: int = 16) -> d
     return out
 
 
-def _window_splits(cache, window: int) -> int:
-    """Key splits of a decode step: the cache's count, but no more than the window has 64-key pieces."""
+def _window_splits(cache, window: int, per: int = 64) -> int:
+    """Key splits of a decode step: one per ``per`` keys that a query can reach (its window, or the cache), at most 32.
+    Fixed per cache and layer, so a captured decode step keeps its launch shapes."""
     reach = min(window or cache.max_len, cache.max_len)
-    return max(1, min(cache.decode_splits, (reach + 63) // 64))
+    return max(1, min(32, (reach + per - 1) // per))
 
 
 class WindowLatentAttentionMixer(_Sublayer):
@@ -212,8 +214,9 @@ class WindowLatentAttentionMixer(_Sublayer):
         a += R + dr
         q_abs = torch.bmm(q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1), self.w_uk)      # [H, T, R]
         oc = latent_attention(q_abs, q, st["ckv"], None, self.inv_freq, H, dn, self.rot_dims, self.scale, sb,
-                              _window_splits(sb.cache, self.window) if sb.decode else 1, True, self.mag, self.window,
-                              self.sinks)                                                    # [T, H, R]
+                              _window_splits(sb.cache, self.window, 32) if sb.decode else 1, True, self.mag,
+                              self.window, self.sinks)                                       # [T, H, R]
+        # (all heads sweep the same rows, so a decode step has few blocks: a split per 32 keys)
         ov = torch.bmm(oc.transpose(0, 1), self.w_uv)                                        # [H, T, dv]
         o = sigmoid_gate(ov.transpose(0, 1).reshape(T, H * self.dv), P[:, a:a + H * self.dv])
         return o @ self.w_o.t()
