@@ -27,7 +27,7 @@ SIZES = {
 def mamivik_config(s: dict, ff: int, vocab: int = 32000) -> dict:
     def par():
         left = {"heads": s["lh"], "kv_heads": s["lg"], "dim": s["ld"], "vdim": s["ld"], "scale": s["ld"] ** -0.5,
-                "mask": {"size": s["window"]}, "rot": {"base": 1e6, "dims": s["lrot"]}}
+                "mask": {"size": s["window"]}, "rot": {"base": 500000.0, "dims": s["lrot"]}}
         return {"type": "parallel", "mixer": {"left": left, "right": {"heads": s["rh"], "dim": s["rd"]},
                                               "left_scale": 1.0, "right_scale": 1.0}}
 

@@ -558,7 +558,7 @@ def test_bf16_matrix_core_sizes_long_context(device, heads, kv_heads, window):
     """Sizes the matrix-core sweeps take (four heads per kv head, one, three), 300 keys, windows inside and across
     tiles, decode with key splits; latent rows of 128 and 64 columns."""
     cfg = config([par(heads=heads, kv_heads=kv_heads, dim=32, rot=16, window=window, rheads=2, rdim=32, scale=0.1, mlp=dense()),
-                  latent(heads=heads, dim=16, rot_dim=32, vdim=24, kv_rank=96, q_rank=24, window=window, scale=0.08, mlp=dense()),
+                  latent(heads=heads, dim=16, rot_dim=64, vdim=24, kv_rank=64, q_rank=24, window=window, scale=0.08, mlp=dense()),
                   par(heads=heads, kv_heads=kv_heads, dim=64, rot=64, window=window + 7, rheads=1, rdim=64, scale=0.06),
                   latent(heads=heads // kv_heads, dim=8, rot_dim=32, vdim=16, kv_rank=32, q_rank=16, window=window + 1, scale=0.08)],
                  width=64)
