@@ -431,16 +431,18 @@ __global__ __launch_bounds__(256) void k_gdr_scan(const T* __restrict__ q, int l
     __syncthreads();
     if (c0 + CT < t1) fetch(c0 + CT);
     // the dot product k . s of a token runs in the same sweep as the read-out of the token before it (both read the
-    // new s), so only the chunk's first token needs a sweep of its own.  Every row vector is read from LDS where it
-    // is used (no register copies from token to token: the scan is bound by its vector instructions).
+    // new s), so only the chunk's first token needs a sweep of its own.  The scan is bound by the bytes its LDS reads
+    // move: a token's key is read once (as the next key of the token before it) and kept in registers; the loop runs
+    // two tokens per turn so that the two register sets swap roles without copies.
+    f32x4 ka_[KR / 4], kb_[KR / 4];
     float dot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i4 = 0; i4 < KR / 4; ++i4) {
-      const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + l0 + 4 * i4);
+      ka_[i4] = *reinterpret_cast<const f32x4*>(sk + l0 + 4 * i4);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dot[j] += Sr[4 * i4 + j] * kk[j];
+      for (int j = 0; j < 4; ++j) dot[j] += Sr[4 * i4 + j] * ka_[i4][j];
     }
-    for (int tt = 0; tt < n; ++tt) {
+    auto step = [&](int tt, const f32x4 (&kk)[KR / 4], f32x4 (&kn)[KR / 4]) {
       const int tn = min(tt + 1, n - 1);
       const float e = sb[tt] * group_sum<R>((dot[0] + dot[1]) + (dot[2] + dot[3]));
       const float vv = sv[tt * NC + cl];
@@ -449,22 +451,27 @@ __global__ __launch_bounds__(256) void k_gdr_scan(const T* __restrict__ q, int l
       for (int j = 0; j < 4; ++j) dot[j] = 0.f;
 #pragma unroll
       for (int i4 = 0; i4 < KR / 4; ++i4) {
-        const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + tt * LDR + l0 + 4 * i4);
         const f32x4 wd = *reinterpret_cast<const f32x4*>(sd + tt * LDR + l0 + 4 * i4);
         const f32x4 ka = *reinterpret_cast<const f32x4*>(sa + tt * LDR + l0 + 4 * i4);
         const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * LDR + l0 + 4 * i4);
-        const f32x4 kn = *reinterpret_cast<const f32x4*>(sk + tn * LDR + l0 + 4 * i4);
+        kn[i4] = *reinterpret_cast<const f32x4*>(sk + tn * LDR + l0 + 4 * i4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float sn = (wd[j] * Sr[4 * i4 + j] + kk[j] * vv) - ka[j] * e;
+          const float sn = (wd[j] * Sr[4 * i4 + j] + kk[i4][j] * vv) - ka[j] * e;
           Sr[4 * i4 + j] = sn;
           o[j] += sn * qq[j];
-          dot[j] += sn * kn[j];
+          dot[j] += sn * kn[i4][j];
         }
       }
       const float ov = group_sum<R>((o[0] + o[1]) + (o[2] + o[3]));
       if (rg == 0 && colok) out[((size_t)(c0 + tt) * H + hd) * dv + col] = ov;
+    };
+    int tt = 0;
+    for (; tt + 1 < n; tt += 2) {
+      step(tt, ka_, kb_);
+      step(tt + 1, kb_, ka_);
     }
+    if (tt < n) step(tt, ka_, kb_);
   }
   if (colok) store_rows(Sp, r0, dk, Sr);
 }
